@@ -1,0 +1,161 @@
+/*
+ * lutgemm_c.h -- C ABI of the MI355X (gfx950) LUT-GEMM library (liblutgemm_hip.so).
+ *
+ * Plain pointers and sizes only; every function returns a lutgemm_status.  The C++ API of
+ * the reference (namespace lutGEMM, headers "lutGEMM", "kernels.h", "nQWeight_fp16.h" in
+ * this directory) is a header-only layer over these entry points.
+ *
+ * Citations name the interface of the reference tree that each entry point stands in for.
+ *
+ * Host-side input layout of a BCQ weight (identical to the reference's, so a caller's
+ * existing packer keeps working):
+ *   bW     uint32 [k/32][q][n]   bit t of bW[w][b][j] is the sign of weight (32 w + t, j) in
+ *                                plane b, 1 = +1, 0 = -1
+ *   alpha  float  [num_groups][q][n]   per-group scale, group length g = k / num_groups
+ *   q_bias float  [num_groups][n] or NULL   per-group additive offset
+ *   W[i][j] = sum_b alpha[i/g][b][j] * sign(b,i,j) + q_bias[i/g][j];   y[j] = sum_i x[i] W[i][j]
+ * Inside the handle the planes are re-tiled for 64-lane wavefronts; the device layout is
+ * private to the library.
+ */
+#ifndef LUTGEMM_C_H
+#define LUTGEMM_C_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef enum lutgemm_status {
+    LUTGEMM_OK = 0,
+    LUTGEMM_ERR_NULL_POINTER = 1,  /* a required pointer argument is NULL */
+    LUTGEMM_ERR_BAD_SHAPE = 2,     /* k, n, q, num_groups or m violate the preconditions */
+    LUTGEMM_ERR_NO_DEVICE = 3,     /* no HIP device / the device is not usable */
+    LUTGEMM_ERR_HIP = 4,           /* a HIP runtime call failed; see lutgemm_last_error() */
+    LUTGEMM_ERR_OUT_OF_MEMORY = 5, /* host or device allocation failed */
+    LUTGEMM_ERR_UNSUPPORTED = 6    /* valid request outside what this build implements */
+} lutgemm_status;
+
+/* Opaque packed weight: device-resident sign tiles, scales and offsets plus the launch plan
+ * and the split-K workspace.  Stands in for class lutGEMM::nQWeight_fp16
+ * (lutGEMM/include/nQWeight_fp16.h:27-52). */
+typedef struct lutgemm_weight lutgemm_weight;
+
+/* Shape record returned by lutgemm_weight_info(); field meanings follow the public data
+ * members of nQWeight_fp16 (lutGEMM/include/nQWeight_fp16.h:29-37). */
+typedef struct lutgemm_weight_info_t {
+    int k;            /* kSize: reduction length */
+    int n;            /* mSize: number of outputs */
+    int q;            /* nb: bit-planes */
+    int num_groups;   /* num_groups */
+    int group_size;   /* k / num_groups */
+    int has_offset;   /* q_bias != nullptr */
+    size_t sign_bytes;   /* k*n*q/8: packed sign bytes streamed per matvec (unpadded) */
+    size_t scale_bytes;  /* num_groups*q*n*2 (unpadded) */
+    size_t offset_bytes; /* num_groups*n*2 or 0 (unpadded) */
+    size_t device_bytes; /* bytes of device memory held by the handle, workspace included */
+} lutgemm_weight_info_t;
+
+/* Build a packed weight from HOST arrays in the layout above (floats are rounded to fp16,
+ * round-to-nearest-even).  Replaces nQWeight_fp16::parsing with is_row_wise_quantize=false
+ * (lutGEMM/src/nQWeight_fp16.cu:60-91): same inputs, but the sign planes are re-tiled for
+ * coalesced wave64 reads instead of being copied verbatim.
+ * Preconditions (LUTGEMM_ERR_BAD_SHAPE otherwise): k > 0, k % 32 == 0, n > 0, 1 <= q <= 8,
+ * num_groups >= 1, k % num_groups == 0 and (k / num_groups) % 32 == 0.
+ * The handle lives on the current HIP device. */
+int lutgemm_weight_create(const uint32_t *bW, const float *alpha, const float *q_bias, int k, int n,
+                          int q, int num_groups, lutgemm_weight **out);
+
+/* As above with alpha / q_bias already in fp16 (host arrays of binary16 bit patterns). */
+int lutgemm_weight_create_f16(const uint32_t *bW, const uint16_t *alpha, const uint16_t *q_bias,
+                              int k, int n, int q, int num_groups, lutgemm_weight **out);
+
+/* Free everything the handle owns, each allocation exactly once; NULL is accepted.
+ * Replaces nQWeight_fp16::~nQWeight_fp16 (lutGEMM/src/nQWeight_fp16.cu:101-105). */
+int lutgemm_weight_destroy(lutgemm_weight *w);
+
+int lutgemm_weight_info(const lutgemm_weight *w, lutgemm_weight_info_t *info);
+
+/* y[r][0..n) = x[r][0..k) * W for r < m, fp16 in / fp16 out, fp32 accumulation, asynchronous
+ * on `stream` (a hipStream_t passed as void*, NULL = the default stream).  x and y are
+ * device pointers, row-major [m][k] and [m][n].  The offset term is applied iff the weight
+ * was created with q_bias.  No memset of y is needed and none is issued.
+ * Replaces lutGEMM::matmul(void* output, void* input, nQWeight_fp16&, int m, int algo)
+ * (lutGEMM/include/kernels.h:27, lutGEMM/src/kernels.cu:64-71), which for m == 1 runs
+ * kernel::nqmv (mv_fp16.hpp:121) or kernel::nqmv_bias (mv_fp16_bias.hpp:143); here every
+ * 1 <= m <= LUTGEMM_MAX_BATCH stays on the table-lookup kernel.
+ * Calls that overlap in time on the same handle race on its split-K workspace. */
+#define LUTGEMM_MAX_BATCH 64
+int lutgemm_matvec(const lutgemm_weight *w, const void *x, void *y, int m, void *stream);
+
+/* Column-batched form: x is [k][m] and y is [n][m] (m vectors stored as columns).
+ * Replaces lutGEMM::matmul(void* output, nQWeight_fp16&, void* input, int n, int algo)
+ * (lutGEMM/include/kernels.h:26, lutGEMM/src/kernels.cu:56-63).  For m == 1 it is the same
+ * operation as lutgemm_matvec. */
+int lutgemm_matvec_cols(const lutgemm_weight *w, const void *x, void *y, int m, void *stream);
+
+/* `count` independent matvecs issued back to back on one stream with a single call (for a
+ * decoder layer's chain of projections, or a benchmark loop): entry i computes
+ * ys[i] = xs[i] * ws[i] with batch ms[i] exactly as lutgemm_matvec would.  Has no counterpart in
+ * the reference, whose caller loops over lutGEMM::matmul itself
+ * (tests/opt/fp16/int3_col_wise_matmul_fp16.cu:120-133).  Stops at the first failing entry. */
+int lutgemm_matvec_many(const lutgemm_weight *const *ws, const void *const *xs, void *const *ys,
+                        const int *ms, int count, void *stream);
+
+/* Dense fp16 weight on the device, W[k][n] (transposed == 0) or W[n][k] (transposed != 0),
+ * offset included.  d_fW is a device pointer to k*n halves.  Asynchronous on `stream`.
+ * Replaces lutGEMM::dequantize_gpu (lutGEMM/src/nQWeight_fp16.cu:29-35); unlike it, the
+ * group index is taken per weight and the offset is not dropped. */
+int lutgemm_dequantize(const lutgemm_weight *w, void *d_fW, int transposed, void *stream);
+
+/* Copy the packed planes back into the host input layout (exact inverse of the re-tiling):
+ * bW [k/32][q][n] uint32, alpha [num_groups][q][n] and q_bias [num_groups][n] as binary16
+ * bit patterns; any output pointer may be NULL to skip it.  Synchronous. */
+int lutgemm_weight_unpack(const lutgemm_weight *w, uint32_t *bW, uint16_t *alpha, uint16_t *q_bias);
+
+/* Launch plan chosen for the handle (for benchmarks and tests): workgroup count, waves per
+ * workgroup, k-splits and 512-wide k-blocks per workgroup. */
+int lutgemm_weight_plan(const lutgemm_weight *w, int *workgroups, int *waves_per_group,
+                        int *k_splits, int *k_blocks_per_group);
+
+/* Override the launch plan (0 keeps the automatic choice for that field); reallocates the
+ * split-K workspace.  Returns LUTGEMM_ERR_BAD_SHAPE if the request cannot be launched. */
+int lutgemm_weight_set_plan(lutgemm_weight *w, int waves_per_group, int k_splits);
+
+/* Device pointers of the packed arrays, for the public data members of the C++ layer. */
+int lutgemm_weight_device_ptrs(const lutgemm_weight *w, void **signs, void **scales, void **offsets);
+
+/* ---- Host-only packer entry points: no HIP device is touched ------------------------------
+ * The re-tiling that lutgemm_weight_create performs, exposed for offline packing and for tests.
+ * They stand where the reference has a verbatim cudaMemcpy of the planes
+ * (lutGEMM/src/nQWeight_fp16.cu:87-88). */
+
+/* Bytes of the sign tiles and of the scale tiles (scales and offsets interleaved) for a shape. */
+int lutgemm_packed_sizes(int k, int n, int q, int num_groups, int has_offset, size_t *sign_bytes,
+                         size_t *scale_bytes);
+
+/* Host input layout -> device tiles, into caller-provided host buffers of the sizes above.
+ * alpha / q_bias are binary16 bit patterns; q_bias may be NULL. */
+int lutgemm_pack_host(const uint32_t *bW, const uint16_t *alpha, const uint16_t *q_bias, int k, int n,
+                      int q, int num_groups, void *signs_out, void *scales_out);
+
+/* Exact inverse of lutgemm_pack_host; any of bW / alpha / q_bias may be NULL. */
+int lutgemm_unpack_host(const void *signs, const void *scales, int k, int n, int q, int num_groups,
+                        int has_offset, uint32_t *bW, uint16_t *alpha, uint16_t *q_bias);
+
+/* float -> binary16 bit patterns, round to nearest even: the conversion applied to alpha and
+ * q_bias at ingest (stands for the __float2half loops of lutGEMM/src/nQWeight_fp16.cu:81,85). */
+int lutgemm_float_to_half(const float *src, uint16_t *dst, size_t count);
+
+/* Thread-local text of the last failure in this library ("" if none). */
+const char *lutgemm_last_error(void);
+const char *lutgemm_status_string(int status);
+
+/* Library / build identification, e.g. "lutgemm-hip gfx950". */
+const char *lutgemm_version(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* LUTGEMM_C_H */

@@ -1,0 +1,455 @@
+// C ABI host layer (include/lutgemm_c.h): argument checks, packing, device memory, launch
+// planning and kernel dispatch.  Calls the HIP runtime directly.
+#include "../../include/lutgemm_c.h"
+
+#include <hip/hip_runtime_api.h>
+
+#include <cstdarg>
+#include <cstdio>
+#include <cstring>
+#include <new>
+#include <vector>
+
+#include "kernels.h"
+#include "layout.h"
+#include "packer.h"
+
+using namespace lutgemm_layout;
+
+namespace {
+
+thread_local char g_error[512] = "";
+
+int fail(int status, const char *fmt, ...)
+{
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_error, sizeof(g_error), fmt, ap);
+    va_end(ap);
+    return status;
+}
+
+int hip_fail(hipError_t e, const char *what)
+{
+    return fail(e == hipErrorOutOfMemory ? LUTGEMM_ERR_OUT_OF_MEMORY : LUTGEMM_ERR_HIP, "%s: %s (%d)",
+                what, hipGetErrorString(e), (int)e);
+}
+
+constexpr int kMaxWaves = 12;  // the kernel is compiled for at most 768 threads per workgroup
+
+struct Plan {
+    int waves;             // wavefronts (= output batches) per workgroup
+    int ntiles;            // column tiles
+    int blocks_per_split;  // k-blocks per workgroup
+    int k_splits;          // workgroups along k
+};
+
+}  // namespace
+
+struct lutgemm_weight {
+    Shape shape;
+    int device;
+    int compute_units;
+    uint8_t *d_signs;
+    uint16_t *d_scales;
+    float *d_partials;
+    unsigned *d_counters;
+    size_t partial_bytes, counter_bytes;
+    Plan plan;
+};
+
+namespace {
+
+// Choose waves per workgroup and the k-split so that the workgroups fill the compute units
+// in as few, as full rounds as possible.  One workgroup owns `waves` batches of 32 outputs
+// and `blocks_per_split` k-blocks; it rebuilds one 64 KiB table set per k-block, so more
+// waves per workgroup amortise the build, and more k-blocks per workgroup amortise the final
+// cross-lane reduction and the split-k exchange.
+Plan choose_plan(const Shape &s, int cus)
+{
+    Plan best{};
+    double best_cost = 1e300;
+    // rough per-workgroup costs in SIMD issue slots (wave instructions per SIMD)
+    const double lookup = 2.0 * s.q * 16 * 3.2 + (s.has_offset ? 40 : 0);
+    for (int waves = 1; waves <= kMaxWaves; waves++) {
+        const int ntiles = div_up(s.nb, waves);
+        const double per_simd = (double)div_up(waves, 4);
+        for (int splits = 1; splits <= s.ts; splits++) {
+            const int bps = div_up(s.ts, splits);
+            const int ks = div_up(s.ts, bps);
+            if (ks != splits) continue;  // same plan as a smaller `splits`
+            const long wgs = (long)ntiles * ks;
+            const double rounds = (double)((wgs + cus - 1) / cus);
+            const double build = 160.0 + 40.0;  // quarter build + barriers
+            double wg_cost = bps * (build + per_simd * lookup) + per_simd * 180.0;
+            if (ks > 1) wg_cost += 300.0;  // fence + ticket + partial traffic
+            // padding waste: wavefronts beyond the last batch still stream a tile
+            const double cost = rounds * wg_cost;
+            if (cost < best_cost - 1e-9) {
+                best_cost = cost;
+                best = Plan{waves, ntiles, bps, ks};
+            }
+        }
+    }
+    return best;
+}
+
+int alloc_workspace(lutgemm_weight *w)
+{
+    if (w->d_partials) (void)hipFree(w->d_partials);
+    if (w->d_counters) (void)hipFree(w->d_counters);
+    w->d_partials = nullptr;
+    w->d_counters = nullptr;
+    w->partial_bytes = (size_t)w->plan.k_splits * w->shape.nb * kBatch * sizeof(float);
+    w->counter_bytes = (size_t)w->plan.ntiles * sizeof(unsigned);
+    hipError_t e = hipMalloc((void **)&w->d_partials, w->partial_bytes);
+    if (e != hipSuccess) return hip_fail(e, "hipMalloc(partials)");
+    e = hipMalloc((void **)&w->d_counters, w->counter_bytes);
+    if (e != hipSuccess) return hip_fail(e, "hipMalloc(counters)");
+    e = hipMemset(w->d_counters, 0, w->counter_bytes);
+    if (e != hipSuccess) return hip_fail(e, "hipMemset(counters)");
+    return LUTGEMM_OK;
+}
+
+int create_common(const uint32_t *bW, const uint16_t *alpha_h, const uint16_t *q_bias_h, int k, int n,
+                  int q, int num_groups, lutgemm_weight **out)
+{
+    Shape s;
+    if (!make_shape(k, n, q, num_groups, q_bias_h != nullptr, &s))
+        return fail(LUTGEMM_ERR_BAD_SHAPE,
+                    "bad shape k=%d n=%d q=%d num_groups=%d (need k%%32==0, 1<=q<=8, "
+                    "k%%num_groups==0, (k/num_groups)%%32==0)",
+                    k, n, q, num_groups);
+    int count = 0;
+    hipError_t e = hipGetDeviceCount(&count);
+    if (e != hipSuccess || count <= 0)
+        return fail(LUTGEMM_ERR_NO_DEVICE, "no HIP device available (%s)",
+                    e == hipSuccess ? "device count is 0" : hipGetErrorString(e));
+    int dev = 0;
+    e = hipGetDevice(&dev);
+    if (e != hipSuccess) return hip_fail(e, "hipGetDevice");
+    hipDeviceProp_t prop;
+    e = hipGetDeviceProperties(&prop, dev);
+    if (e != hipSuccess) return hip_fail(e, "hipGetDeviceProperties");
+
+    lutgemm_weight *w = new (std::nothrow) lutgemm_weight();
+    if (!w) return fail(LUTGEMM_ERR_OUT_OF_MEMORY, "host allocation failed");
+    w->shape = s;
+    w->device = dev;
+    w->compute_units = prop.multiProcessorCount > 0 ? prop.multiProcessorCount : 256;
+
+    const size_t sb = sign_bytes(s), cb = scale_bytes(s);
+    std::vector<uint8_t> signs;
+    std::vector<uint16_t> scales;
+    try {
+        signs.resize(sb);
+        scales.resize(cb / 2);
+    } catch (const std::bad_alloc &) {
+        delete w;
+        return fail(LUTGEMM_ERR_OUT_OF_MEMORY, "host staging allocation failed (%zu bytes)", sb + cb);
+    }
+    lutgemm_packer::pack(s, bW, alpha_h, q_bias_h, signs.data(), scales.data());
+
+    int st = LUTGEMM_OK;
+    e = hipMalloc((void **)&w->d_signs, sb);
+    if (e != hipSuccess) st = hip_fail(e, "hipMalloc(signs)");
+    if (st == LUTGEMM_OK) {
+        e = hipMalloc((void **)&w->d_scales, cb);
+        if (e != hipSuccess) st = hip_fail(e, "hipMalloc(scales)");
+    }
+    if (st == LUTGEMM_OK) {
+        e = hipMemcpy(w->d_signs, signs.data(), sb, hipMemcpyHostToDevice);
+        if (e != hipSuccess) st = hip_fail(e, "hipMemcpy(signs)");
+    }
+    if (st == LUTGEMM_OK) {
+        e = hipMemcpy(w->d_scales, scales.data(), cb, hipMemcpyHostToDevice);
+        if (e != hipSuccess) st = hip_fail(e, "hipMemcpy(scales)");
+    }
+    if (st == LUTGEMM_OK) {
+        w->plan = choose_plan(s, w->compute_units);
+        st = alloc_workspace(w);
+    }
+    if (st != LUTGEMM_OK) {
+        lutgemm_weight_destroy(w);
+        return st;
+    }
+    *out = w;
+    return LUTGEMM_OK;
+}
+
+int run_matvec(const lutgemm_weight *w, const void *x, void *y, int m, void *stream, bool cols)
+{
+    if (!w || !x || !y) return fail(LUTGEMM_ERR_NULL_POINTER, "null argument to matvec");
+    if (m < 1 || m > LUTGEMM_MAX_BATCH)
+        return fail(LUTGEMM_ERR_BAD_SHAPE, "m=%d outside 1..%d", m, LUTGEMM_MAX_BATCH);
+    const Shape &s = w->shape;
+    lutgemm_kernels::MatvecArgs a{};
+    a.signs = w->d_signs;
+    a.scales = w->d_scales;
+    a.partials = w->d_partials;
+    a.counters = w->d_counters;
+    a.k = s.k;
+    a.n = s.n;
+    a.ts = s.ts;
+    a.nb = s.nb;
+    a.ntiles = w->plan.ntiles;
+    a.k_splits = w->plan.k_splits;
+    a.blocks_per_split = w->plan.blocks_per_split;
+    const uint16_t *xh = static_cast<const uint16_t *>(x);
+    uint16_t *yh = static_cast<uint16_t *>(y);
+    for (int r = 0; r < m; r++) {
+        if (cols) {  // x [k][m], y [n][m]
+            a.x = xh + r;
+            a.y = yh + r;
+            a.x_stride = m;
+            a.y_stride = m;
+        } else {     // x [m][k], y [m][n]
+            a.x = xh + (size_t)r * s.k;
+            a.y = yh + (size_t)r * s.n;
+            a.x_stride = 1;
+            a.y_stride = 1;
+        }
+        hipError_t e = lutgemm_kernels::launch_matvec(s.q, s.has_offset, s.gsub, a,
+                                                      w->plan.ntiles * w->plan.k_splits, w->plan.waves,
+                                                      static_cast<hipStream_t>(stream));
+        if (e != hipSuccess) return hip_fail(e, "launch lut_matvec_kernel");
+    }
+    return LUTGEMM_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+int lutgemm_weight_create_f16(const uint32_t *bW, const uint16_t *alpha, const uint16_t *q_bias, int k,
+                              int n, int q, int num_groups, lutgemm_weight **out)
+{
+    if (!bW || !alpha || !out) return fail(LUTGEMM_ERR_NULL_POINTER, "null argument to weight_create");
+    *out = nullptr;
+    return create_common(bW, alpha, q_bias, k, n, q, num_groups, out);
+}
+
+int lutgemm_weight_create(const uint32_t *bW, const float *alpha, const float *q_bias, int k, int n, int q,
+                          int num_groups, lutgemm_weight **out)
+{
+    if (!bW || !alpha || !out) return fail(LUTGEMM_ERR_NULL_POINTER, "null argument to weight_create");
+    *out = nullptr;
+    Shape s;
+    if (!make_shape(k, n, q, num_groups, q_bias != nullptr, &s))
+        return fail(LUTGEMM_ERR_BAD_SHAPE,
+                    "bad shape k=%d n=%d q=%d num_groups=%d (need k%%32==0, 1<=q<=8, "
+                    "k%%num_groups==0, (k/num_groups)%%32==0)",
+                    k, n, q, num_groups);
+    std::vector<uint16_t> ah, zh;
+    try {
+        ah.resize((size_t)num_groups * q * n);
+        if (q_bias) zh.resize((size_t)num_groups * n);
+    } catch (const std::bad_alloc &) {
+        return fail(LUTGEMM_ERR_OUT_OF_MEMORY, "host allocation failed");
+    }
+    lutgemm_packer::floats_to_halves(alpha, ah.data(), ah.size());
+    if (q_bias) lutgemm_packer::floats_to_halves(q_bias, zh.data(), zh.size());
+    return create_common(bW, ah.data(), q_bias ? zh.data() : nullptr, k, n, q, num_groups, out);
+}
+
+int lutgemm_weight_destroy(lutgemm_weight *w)
+{
+    if (!w) return LUTGEMM_OK;
+    int st = LUTGEMM_OK;
+    void *ptrs[4] = {w->d_signs, w->d_scales, w->d_partials, w->d_counters};
+    for (void *p : ptrs)
+        if (p) {
+            hipError_t e = hipFree(p);
+            if (e != hipSuccess) st = hip_fail(e, "hipFree");
+        }
+    delete w;
+    return st;
+}
+
+int lutgemm_weight_info(const lutgemm_weight *w, lutgemm_weight_info_t *info)
+{
+    if (!w || !info) return fail(LUTGEMM_ERR_NULL_POINTER, "null argument to weight_info");
+    const Shape &s = w->shape;
+    info->k = s.k;
+    info->n = s.n;
+    info->q = s.q;
+    info->num_groups = s.num_groups;
+    info->group_size = s.group_size;
+    info->has_offset = s.has_offset;
+    info->sign_bytes = (size_t)s.k / 8 * s.q * s.n;
+    info->scale_bytes = (size_t)s.num_groups * s.q * s.n * 2;
+    info->offset_bytes = s.has_offset ? (size_t)s.num_groups * s.n * 2 : 0;
+    info->device_bytes = sign_bytes(s) + scale_bytes(s) + w->partial_bytes + w->counter_bytes;
+    return LUTGEMM_OK;
+}
+
+int lutgemm_matvec(const lutgemm_weight *w, const void *x, void *y, int m, void *stream)
+{
+    return run_matvec(w, x, y, m, stream, false);
+}
+
+int lutgemm_matvec_cols(const lutgemm_weight *w, const void *x, void *y, int m, void *stream)
+{
+    return run_matvec(w, x, y, m, stream, true);
+}
+
+int lutgemm_matvec_many(const lutgemm_weight *const *ws, const void *const *xs, void *const *ys,
+                        const int *ms, int count, void *stream)
+{
+    if (!ws || !xs || !ys || !ms) return fail(LUTGEMM_ERR_NULL_POINTER, "null argument to matvec_many");
+    if (count < 0) return fail(LUTGEMM_ERR_BAD_SHAPE, "count=%d is negative", count);
+    for (int i = 0; i < count; i++) {
+        int st = run_matvec(ws[i], xs[i], ys[i], ms[i], stream, false);
+        if (st != LUTGEMM_OK) return st;
+    }
+    return LUTGEMM_OK;
+}
+
+int lutgemm_dequantize(const lutgemm_weight *w, void *d_fW, int transposed, void *stream)
+{
+    if (!w || !d_fW) return fail(LUTGEMM_ERR_NULL_POINTER, "null argument to dequantize");
+    const Shape &s = w->shape;
+    lutgemm_kernels::DequantArgs a{};
+    a.signs = w->d_signs;
+    a.scales = w->d_scales;
+    a.out = d_fW;
+    a.k = s.k;
+    a.n = s.n;
+    a.q = s.q;
+    a.has_offset = s.has_offset;
+    a.gsub = s.gsub;
+    a.ts = s.ts;
+    a.transposed = transposed ? 1 : 0;
+    hipError_t e = lutgemm_kernels::launch_dequantize(a, static_cast<hipStream_t>(stream));
+    if (e != hipSuccess) return hip_fail(e, "launch dequantize_kernel");
+    return LUTGEMM_OK;
+}
+
+int lutgemm_weight_unpack(const lutgemm_weight *w, uint32_t *bW, uint16_t *alpha, uint16_t *q_bias)
+{
+    if (!w) return fail(LUTGEMM_ERR_NULL_POINTER, "null argument to weight_unpack");
+    const Shape &s = w->shape;
+    std::vector<uint8_t> signs;
+    std::vector<uint16_t> scales;
+    try {
+        signs.resize(sign_bytes(s));
+        scales.resize(scale_bytes(s) / 2);
+    } catch (const std::bad_alloc &) {
+        return fail(LUTGEMM_ERR_OUT_OF_MEMORY, "host staging allocation failed");
+    }
+    hipError_t e = hipMemcpy(signs.data(), w->d_signs, signs.size(), hipMemcpyDeviceToHost);
+    if (e != hipSuccess) return hip_fail(e, "hipMemcpy(signs)");
+    e = hipMemcpy(scales.data(), w->d_scales, scales.size() * 2, hipMemcpyDeviceToHost);
+    if (e != hipSuccess) return hip_fail(e, "hipMemcpy(scales)");
+    lutgemm_packer::unpack(s, signs.data(), scales.data(), bW, alpha, s.has_offset ? q_bias : nullptr);
+    return LUTGEMM_OK;
+}
+
+int lutgemm_weight_plan(const lutgemm_weight *w, int *workgroups, int *waves_per_group, int *k_splits,
+                        int *k_blocks_per_group)
+{
+    if (!w) return fail(LUTGEMM_ERR_NULL_POINTER, "null argument to weight_plan");
+    if (workgroups) *workgroups = w->plan.ntiles * w->plan.k_splits;
+    if (waves_per_group) *waves_per_group = w->plan.waves;
+    if (k_splits) *k_splits = w->plan.k_splits;
+    if (k_blocks_per_group) *k_blocks_per_group = w->plan.blocks_per_split;
+    return LUTGEMM_OK;
+}
+
+int lutgemm_weight_set_plan(lutgemm_weight *w, int waves_per_group, int k_splits)
+{
+    if (!w) return fail(LUTGEMM_ERR_NULL_POINTER, "null argument to weight_set_plan");
+    const Shape &s = w->shape;
+    Plan p = choose_plan(s, w->compute_units);
+    if (waves_per_group != 0) {
+        if (waves_per_group < 1 || waves_per_group > kMaxWaves)
+            return fail(LUTGEMM_ERR_BAD_SHAPE, "waves_per_group=%d outside 1..%d", waves_per_group, kMaxWaves);
+        p.waves = waves_per_group;
+        p.ntiles = div_up(s.nb, p.waves);
+    }
+    if (k_splits != 0) {
+        if (k_splits < 1 || k_splits > s.ts)
+            return fail(LUTGEMM_ERR_BAD_SHAPE, "k_splits=%d outside 1..%d", k_splits, s.ts);
+        p.blocks_per_split = div_up(s.ts, k_splits);
+        p.k_splits = div_up(s.ts, p.blocks_per_split);
+    }
+    hipError_t e = hipDeviceSynchronize();  // no launch may still be using the old workspace
+    if (e != hipSuccess) return hip_fail(e, "hipDeviceSynchronize");
+    w->plan = p;
+    return alloc_workspace(w);
+}
+
+int lutgemm_weight_device_ptrs(const lutgemm_weight *w, void **signs, void **scales, void **offsets)
+{
+    if (!w) return fail(LUTGEMM_ERR_NULL_POINTER, "null argument to weight_device_ptrs");
+    if (signs) *signs = w->d_signs;
+    if (scales) *scales = w->d_scales;
+    // offsets are interleaved with the scales in the scale tiles; non-null iff present
+    if (offsets) *offsets = w->shape.has_offset ? (void *)w->d_scales : nullptr;
+    return LUTGEMM_OK;
+}
+
+/* ---- host-only packer entry points (no device needed) ---- */
+
+int lutgemm_packed_sizes(int k, int n, int q, int num_groups, int has_offset, size_t *sign_bytes_out,
+                         size_t *scale_bytes_out)
+{
+    Shape s;
+    if (!make_shape(k, n, q, num_groups, has_offset, &s))
+        return fail(LUTGEMM_ERR_BAD_SHAPE, "bad shape k=%d n=%d q=%d num_groups=%d", k, n, q, num_groups);
+    if (sign_bytes_out) *sign_bytes_out = sign_bytes(s);
+    if (scale_bytes_out) *scale_bytes_out = scale_bytes(s);
+    return LUTGEMM_OK;
+}
+
+int lutgemm_pack_host(const uint32_t *bW, const uint16_t *alpha, const uint16_t *q_bias, int k, int n, int q,
+                      int num_groups, void *signs_out, void *scales_out)
+{
+    if (!bW || !alpha || !signs_out || !scales_out)
+        return fail(LUTGEMM_ERR_NULL_POINTER, "null argument to pack_host");
+    Shape s;
+    if (!make_shape(k, n, q, num_groups, q_bias != nullptr, &s))
+        return fail(LUTGEMM_ERR_BAD_SHAPE, "bad shape k=%d n=%d q=%d num_groups=%d", k, n, q, num_groups);
+    lutgemm_packer::pack(s, bW, alpha, q_bias, static_cast<uint8_t *>(signs_out),
+                         static_cast<uint16_t *>(scales_out));
+    return LUTGEMM_OK;
+}
+
+int lutgemm_unpack_host(const void *signs, const void *scales, int k, int n, int q, int num_groups,
+                        int has_offset, uint32_t *bW, uint16_t *alpha, uint16_t *q_bias)
+{
+    if (!signs || !scales) return fail(LUTGEMM_ERR_NULL_POINTER, "null argument to unpack_host");
+    Shape s;
+    if (!make_shape(k, n, q, num_groups, has_offset, &s))
+        return fail(LUTGEMM_ERR_BAD_SHAPE, "bad shape k=%d n=%d q=%d num_groups=%d", k, n, q, num_groups);
+    lutgemm_packer::unpack(s, static_cast<const uint8_t *>(signs), static_cast<const uint16_t *>(scales), bW,
+                           alpha, has_offset ? q_bias : nullptr);
+    return LUTGEMM_OK;
+}
+
+int lutgemm_float_to_half(const float *src, uint16_t *dst, size_t count)
+{
+    if (!src || !dst) return fail(LUTGEMM_ERR_NULL_POINTER, "null argument to float_to_half");
+    lutgemm_packer::floats_to_halves(src, dst, count);
+    return LUTGEMM_OK;
+}
+
+const char *lutgemm_last_error(void) { return g_error; }
+
+const char *lutgemm_status_string(int status)
+{
+    switch (status) {
+        case LUTGEMM_OK: return "ok";
+        case LUTGEMM_ERR_NULL_POINTER: return "null pointer";
+        case LUTGEMM_ERR_BAD_SHAPE: return "bad shape";
+        case LUTGEMM_ERR_NO_DEVICE: return "no device";
+        case LUTGEMM_ERR_HIP: return "HIP runtime error";
+        case LUTGEMM_ERR_OUT_OF_MEMORY: return "out of memory";
+        case LUTGEMM_ERR_UNSUPPORTED: return "unsupported";
+        default: return "unknown status";
+    }
+}
+
+const char *lutgemm_version(void) { return "lutgemm-hip 0.1 gfx950"; }
+
+}  // extern "C"

@@ -1,0 +1,41 @@
+// Launch interface between the C ABI host layer and the gfx950 kernels.
+#ifndef LUTGEMM_KERNELS_H
+#define LUTGEMM_KERNELS_H
+
+#include <hip/hip_runtime_api.h>
+#include <stddef.h>
+#include <stdint.h>
+
+namespace lutgemm_kernels {
+
+struct MatvecArgs {
+    const uint8_t *signs;   // sign tiles (layout.h)
+    const uint16_t *scales; // scale tiles (layout.h)
+    const void *x;          // fp16 activations, element i at x[i * x_stride]
+    void *y;                // fp16 outputs, element j at y[j * y_stride]
+    float *partials;        // [k_splits][nb*32] fp32, used when k_splits > 1
+    unsigned *counters;     // [ntiles] arrival counters, zero between launches
+    int k, n;
+    int ts, nb;             // k-blocks, output batches
+    int ntiles;             // column tiles = ceil(nb / waves)
+    int k_splits;           // workgroups along k
+    int blocks_per_split;   // k-blocks per workgroup
+    int x_stride, y_stride;
+};
+
+struct DequantArgs {
+    const uint8_t *signs;
+    const uint16_t *scales;
+    void *out;              // fp16 [k][n] or [n][k]
+    int k, n, q, has_offset, gsub, ts;
+    int transposed;
+};
+
+// workgroups = ntiles * k_splits, `waves` wavefronts of 64 lanes per workgroup.
+hipError_t launch_matvec(int q, int has_offset, int gsub, const MatvecArgs &a, int workgroups,
+                         int waves, hipStream_t stream);
+
+hipError_t launch_dequantize(const DequantArgs &a, hipStream_t stream);
+
+}  // namespace lutgemm_kernels
+#endif

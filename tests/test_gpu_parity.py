@@ -1,0 +1,198 @@
+"""GPU parity: the HIP library, called through its C ABI, against the CPU oracle on the same
+seeded inputs.  Floating-point path: tolerance stated in gpu_util.py; integer-exact cases
+(unit activations, dequantisation without offset, unpacking) are compared bit for bit."""
+import sys
+
+import numpy as np
+import pytest
+
+from gpu_util import assert_within_tolerance, run_matvec
+
+pytestmark = pytest.mark.gpu
+
+
+def say(*a):
+    print(*a, flush=True)
+    sys.stdout.flush()
+
+
+def make(lg, synth, k, n, q, g, rtn=False, offset=None, seed=0):
+    w = synth.make_weight(k, n, q, g, rtn=rtn, offset=offset, seed=seed)
+    return w, lg.BCQWeight(w["bW"], w["alpha"], k, n, q, k // g, w["q_bias"])
+
+
+def truth_of(oracle, w, x):
+    z = w["q_bias"].astype(np.float16) if w["q_bias"] is not None else None
+    return oracle.matvec_f64(w["bW"], w["alpha"].astype(np.float16), z, x)
+
+
+SMALL = [  # k, n, q, g, offset
+    (512, 32, 3, 128, False), (512, 64, 3, 128, True), (1024, 96, 1, 64, False), (1536, 100, 2, 32, True),
+    (32, 1, 1, 32, False), (96, 33, 4, 96, True), (640, 70, 8, 128, False), (2048, 40, 3, 2048, True),
+    (1024, 17, 5, 256, False), (192, 100, 2, 64, True), (4096, 8, 3, 128, False), (7168, 224, 3, 128, False),
+    (1024, 2048, 4, 128, True), (3072, 1000, 3, 64, False), (2560, 513, 2, 32, False), (512, 4096, 6, 512, True),
+]
+
+
+@pytest.mark.parametrize("k,n,q,g,offset", SMALL)
+def test_small_shapes_match_oracle(lutgemm, oracle, device, k, n, q, g, offset):
+    from lutgemm import synth
+    say("case small", k, n, q, g, offset)
+    w, W = make(lutgemm, synth, k, n, q, g, offset=offset, seed=k + n)
+    x = synth.make_x(1, k, seed=q)
+    y = run_matvec(lutgemm, W, x, device)
+    assert_within_tolerance(y, truth_of(oracle, w, x), "k=%d n=%d q=%d g=%d off=%s plan=%s" % (k, n, q, g, offset, W.plan()))
+    W.close()
+
+
+@pytest.mark.parametrize("q", [1, 2, 3, 4])
+@pytest.mark.parametrize("g", [32, 64, 128, 1792])
+def test_bit_group_sweep(lutgemm, oracle, device, q, g):
+    """The q x g sweep at a quarter of the benchmark's 7168 x 7168 shape (same group modes)."""
+    from lutgemm import synth
+    k = n = 1792
+    say("case sweep", q, g)
+    w, W = make(lutgemm, synth, k, n, q, g, seed=q * 100 + g)
+    x = synth.make_x(1, k, seed=5)
+    assert_within_tolerance(run_matvec(lutgemm, W, x, device), truth_of(oracle, w, x), "q=%d g=%d" % (q, g))
+    W.close()
+
+
+def test_cfg0_and_reference_kernel_error_alongside(lutgemm, oracle, device):
+    from lutgemm import synth
+    c = synth.CONFIGS["cfg0"]
+    say("case cfg0")
+    w, W = make(lutgemm, synth, c["k"], c["n"], c["q"], c["g"], seed=0)
+    x = synth.make_x(1, c["k"], seed=0)
+    truth = truth_of(oracle, w, x)
+    y = run_matvec(lutgemm, W, x, device)
+    assert_within_tolerance(y, truth, "cfg0")
+    ours = oracle.error_stats(y, truth)
+    ref = oracle.error_stats(oracle.ref_kernel_fp16(w["bW"], w["alpha"].astype(np.float16), None, x[0]), truth)
+    say("cfg0 error (mean abs, max abs, rel L2): ours", ours, "emulated reference kernel", ref)
+    assert ours[1] <= ref[1]      # fp32 accumulation is at least as close to the truth as fp16 atomics
+    W.close()
+
+
+def test_cfg1_headline_shape(lutgemm, oracle, device):
+    from lutgemm import synth
+    c = synth.CONFIGS["cfg1"]
+    say("case cfg1")
+    w, W = make(lutgemm, synth, c["k"], c["n"], c["q"], c["g"], seed=1)
+    x = synth.make_x(1, c["k"], seed=1)
+    y = run_matvec(lutgemm, W, x, device)
+    assert_within_tolerance(y, truth_of(oracle, w, x), "cfg1 plan=%s" % W.plan())
+    # determinism: the same launch twice gives bit-identical output
+    y2 = run_matvec(lutgemm, W, x, device)
+    assert np.array_equal(y.view(np.uint16), y2.view(np.uint16))
+    # unit activations: y must be row k of the dequantised weight, bit for bit
+    fW = oracle.dequantize_cpu(w["bW"][:, :, :256], w["alpha"].astype(np.float16)[:, :, :256])
+    for kk in (0, 7, 4095, 12287):
+        e = np.zeros((1, c["k"]), np.float16)
+        e[0, kk] = 1
+        ye = run_matvec(lutgemm, W, e, device)
+        assert np.array_equal(ye[0, :256].view(np.uint16), fW[kk].view(np.uint16)), kk
+    W.close()
+
+
+def test_cfg2_rtn_with_offset_reduced_n(lutgemm, oracle, device):
+    """Uniform 4-bit codes as BCQ with offset, k as in the benchmark, n cut to keep the oracle fast."""
+    from lutgemm import synth
+    say("case cfg2")
+    k, n, q, g = 12288, 4096, 4, 128
+    w, W = make(lutgemm, synth, k, n, q, g, rtn=True, seed=2)
+    x = synth.make_x(1, k, seed=2)
+    truth = truth_of(oracle, w, x)
+    y = run_matvec(lutgemm, W, x, device)
+    assert_within_tolerance(y, truth, "cfg2")
+    # the RTN identity: the same result from the integer codes, y = sum_k x_k s (c - z0) with
+    # s = 2 alpha_0 and s z0 = sum_i alpha_i - offset
+    a16 = w["alpha"].astype(np.float64)
+    codes = np.zeros((k, n), np.int64)
+    for b in range(q):
+        bits = (w["bW"][:, b, :][:, None, :] >> np.arange(32, dtype=np.uint32)[None, :, None]) & 1
+        codes += bits.reshape(k, n).astype(np.int64) << b
+    s = np.repeat(2 * a16[:, 0, :], g, axis=0)
+    sz0 = np.repeat(a16.sum(axis=1) - w["q_bias"].astype(np.float64), g, axis=0)
+    dense = s * codes - sz0
+    assert np.allclose(x.astype(np.float64) @ dense, truth, rtol=1e-9, atol=1e-9)
+    W.close()
+
+
+@pytest.mark.parametrize("m", [2, 4, 8])
+def test_batched_rows_and_columns(lutgemm, oracle, device, m):
+    from lutgemm import synth
+    say("case batch", m)
+    k, n, q, g = 2048, 384, 2, 128
+    w, W = make(lutgemm, synth, k, n, q, g, offset=True, seed=m)
+    x = synth.make_x(m, k, seed=m)
+    truth = truth_of(oracle, w, x)
+    yr = run_matvec(lutgemm, W, x, device)
+    assert_within_tolerance(yr, truth, "rows m=%d" % m)
+    yc = run_matvec(lutgemm, W, x, device, cols=True)
+    assert np.array_equal(yr.view(np.uint16), yc.view(np.uint16))
+    W.close()
+
+
+def test_every_launch_plan_agrees(lutgemm, oracle, device):
+    """Different workgroup shapes / k-splits change the summation order only: all within tolerance,
+    and each plan is deterministic."""
+    from lutgemm import synth
+    k, n, q, g = 4096, 1000, 3, 128
+    w, W = make(lutgemm, synth, k, n, q, g, offset=True, seed=9)
+    x = synth.make_x(1, k, seed=9)
+    truth = truth_of(oracle, w, x)
+    for waves in (1, 3, 4, 7, 12):
+        for ks in (1, 2, 3, 8):
+            say("case plan", waves, ks)
+            W.set_plan(waves, ks)
+            y = run_matvec(lutgemm, W, x, device)
+            assert_within_tolerance(y, truth, "waves=%d ks=%d plan=%s" % (waves, ks, W.plan()))
+            assert np.array_equal(y.view(np.uint16), run_matvec(lutgemm, W, x, device).view(np.uint16))
+    W.close()
+
+
+def test_back_to_back_launches_reuse_workspace(lutgemm, oracle, device):
+    """The split-k arrival counters reset themselves: many launches on one stream stay correct."""
+    import torch
+    from lutgemm import synth
+    k, n, q, g = 4096, 512, 3, 128
+    w, W = make(lutgemm, synth, k, n, q, g, seed=3)
+    W.set_plan(4, 4)
+    xs = synth.make_x(6, k, seed=3)
+    truth = truth_of(oracle, w, xs)
+    xd = torch.from_numpy(xs).to(device)
+    yd = torch.zeros((6, n), dtype=torch.float16, device=device)
+    st = torch.cuda.current_stream().cuda_stream
+    for rep in range(5):
+        for r in range(6):
+            W.matvec(xd[r].data_ptr(), yd[r].data_ptr(), 1, st)
+    torch.cuda.synchronize()
+    assert_within_tolerance(yd.cpu().numpy(), truth, "repeated launches")
+    W.close()
+
+
+def test_device_round_trip_and_dequantize(lutgemm, oracle, device):
+    import torch
+    from lutgemm import synth
+    for (k, n, q, g, off) in [(1024, 100, 3, 128, False), (1536, 70, 2, 64, True), (512, 33, 4, 32, True)]:
+        say("case dequant", k, n, q, g, off)
+        w, W = make(lutgemm, synth, k, n, q, g, offset=off, seed=k)
+        bW, alpha, z = W.unpack()
+        assert np.array_equal(bW, w["bW"])
+        assert np.array_equal(alpha.view(np.uint16), w["alpha"].astype(np.float16).view(np.uint16))
+        if off:
+            assert np.array_equal(z.view(np.uint16), w["q_bias"].astype(np.float16).view(np.uint16))
+        out = torch.empty((k, n), dtype=torch.float16, device=device)
+        out_t = torch.empty((n, k), dtype=torch.float16, device=device)
+        W.dequantize(out.data_ptr(), False, torch.cuda.current_stream().cuda_stream)
+        W.dequantize(out_t.data_ptr(), True, torch.cuda.current_stream().cuda_stream)
+        torch.cuda.synchronize()
+        got = out.cpu().numpy()
+        assert np.array_equal(got, out_t.cpu().numpy().T)
+        if not off:   # same float32 sum order as the reference's CPU dequantisation: bit exact
+            assert np.array_equal(got.view(np.uint16), oracle.dequantize_cpu(w["bW"], w["alpha"].astype(np.float16)).view(np.uint16))
+        dense = oracle.dense_weight_f64(w["bW"], w["alpha"].astype(np.float16),
+                                        w["q_bias"].astype(np.float16) if off else None)
+        assert np.all(np.abs(got.astype(np.float64) - dense) <= 2.0 ** -11 * np.abs(dense) + 2.0 ** -24)
+        W.close()
