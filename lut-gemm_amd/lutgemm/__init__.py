@@ -6,7 +6,8 @@ Mirrors the reference's C++ surface for the BCQ matvec path:
   matmul(output, input, weight, m)                   ~ lutGEMM::matmul(void*, void*, nQWeight_fp16&, int)
                                                       (lutGEMM/src/kernels.cu:64-71)
 Device buffers are passed as integer addresses (e.g. torch.Tensor.data_ptr()); torch is only
-plumbing for device memory and streams and is not imported here.
+plumbing for device memory and streams (it is imported, when present, solely so that both
+share one HIP runtime).
 
 There is no CPU fallback: if the HIP library is missing, loading raises.
 """
@@ -57,6 +58,14 @@ def load():
         raise FileNotFoundError(
             "%s is missing: build it with `make -C %s` (or __graft_entry__.build())"
             % (LIB_PATH, os.path.join(os.path.dirname(_HERE), "csrc")))
+    # One process must use one HIP runtime.  PyTorch-ROCm ships its own libamdhip64 with the
+    # same soname as the system one; importing torch first makes this library bind to the copy
+    # torch uses, so device pointers and streams made by torch are valid here.  Without torch the
+    # system runtime is used.
+    try:
+        import torch  # noqa: F401
+    except ImportError:
+        pass
     L = ctypes.CDLL(LIB_PATH)
     vp, i, sz = ctypes.c_void_p, ctypes.c_int, ctypes.c_size_t
     pp = ctypes.POINTER(ctypes.c_void_p)
