@@ -47,38 +47,133 @@ __device__ __forceinline__ void static_for(F &&body)
     static_for_impl(body, std::make_integer_sequence<int, N>{});
 }
 
-__device__ __forceinline__ float lds_lookup(const float *lds, uint32_t byte_addr)
-{
-    return *reinterpret_cast<const float *>(reinterpret_cast<const char *>(lds) + byte_addr);
-}
+// ------------------------------------------------------------------------------------------
+// Eight table lookups with their scaled accumulation, written in GCN assembly so that a lookup
+// costs two vector ALU instructions and one LDS read:
+//     v_perm_b32      address = {LDS bits 31..16, sign byte, lane * 4} = entry * 256 + lane * 4
+//     ds_read_b32     value   = table[entry][lane]
+//     v_fmac_f32_dpp  acc    += scale (fetched from the lane that holds it) * value
+// The compiler does not fold the cross-lane fetch into the multiply-add by itself and keeps
+// far more lookups in flight than the register budget allows, hence the hand scheduling: all
+// eight reads are issued, then each multiply-add waits only for its own value.
+//
+// Hazard note: a DPP instruction must not read a VGPR that a vector ALU instruction wrote in the
+// two preceding issue slots.  The only DPP-read registers are the scale registers; every block
+// puts at least sixteen other instructions (or an s_nop 1) before its first DPP read, so
+// nothing the compiler places just before a block can violate this.
+//
+// Operands: %0-%7 accumulators, %8-%15 scratch, %16/%17 the two sign dwords, %18 lane offset
+// (its upper half carries LDS address bits 16 and up), %19-%22 byte selectors, %23 (%24) scales.
+// The "memory" clobber keeps the compiler from hoisting the next tiles' global loads above the
+// lookups of the current one, which would double the registers a tile in flight costs.
+// ------------------------------------------------------------------------------------------
+#define LG_ADDR_AND_READ                                                                             \
+    "v_perm_b32 %8, %16, %18, %19\n v_perm_b32 %9, %16, %18, %20\n v_perm_b32 %10, %16, %18, %21\n"   \
+    "v_perm_b32 %11, %16, %18, %22\n v_perm_b32 %12, %17, %18, %19\n v_perm_b32 %13, %17, %18, %20\n" \
+    "v_perm_b32 %14, %17, %18, %21\n v_perm_b32 %15, %17, %18, %22\n"                                 \
+    "ds_read_b32 %8, %8\n ds_read_b32 %9, %9\n ds_read_b32 %10, %10\n ds_read_b32 %11, %11\n"         \
+    "ds_read_b32 %12, %12\n ds_read_b32 %13, %13\n ds_read_b32 %14, %14\n ds_read_b32 %15, %15\n"
+#define LG_OUT(acc, I0, tmp)                                                                          \
+    "+v"(acc[I0 + 0]), "+v"(acc[I0 + 1]), "+v"(acc[I0 + 2]), "+v"(acc[I0 + 3]), "+v"(acc[I0 + 4]),      \
+        "+v"(acc[I0 + 5]), "+v"(acc[I0 + 6]), "+v"(acc[I0 + 7]), "=&v"(tmp[0]), "=&v"(tmp[1]),          \
+        "=&v"(tmp[2]), "=&v"(tmp[3]), "=&v"(tmp[4]), "=&v"(tmp[5]), "=&v"(tmp[6]), "=&v"(tmp[7])
+#define LG_IN(w0, w1, lane_off)                                                                        \
+    "v"(w0), "v"(w1), "v"(lane_off), "s"(0x03020400u), "s"(0x03020500u), "s"(0x03020600u), "s"(0x03020700u)
+#define LG_WAIT(n) "s_waitcnt lgkmcnt(" #n ")\n"
+#define LG_ROW(n) " row_newbcast:" #n " row_mask:0xf bank_mask:0xf\n"
+#define LG_LOHALF(n) " row_newbcast:" #n " row_mask:0xf bank_mask:0x3\n"
+#define LG_HIHALF(n) " row_newbcast:" #n " row_mask:0xf bank_mask:0xc\n"
+#define LG_QUAD(n) " quad_perm:[" #n "," #n "," #n "," #n "] row_mask:0xf bank_mask:0xf\n"
+// multiply-add k of a block: accumulator %k, scale operand S, value %(8+k)
+#define LG_FMA(k, S, v, CTRL) "v_fmac_f32_dpp %" #k ", %" #S ", %" #v CTRL
 
-// a * v + acc with `a` taken from another lane of the same DPP row / half row / quad.
-// CTRL is the DPP control word, BANKS the bank mask (which 4-lane groups of a row take part;
-// the others see a == 0 and leave acc unchanged).
-template <int CTRL, int BANKS>
-__device__ __forceinline__ float fma_bcast(float a, float v, float acc)
+// Outputs I0..I0+7 of the batch (I0 a multiple of 8), sign bytes in w0 (outputs I0..I0+3) and
+// w1 (I0+4..I0+7).  GSUB as in the scale tile layout: the scale of output i sits in
+//   GSUB 1: lane i%16 of the row, in sa
+//   GSUB 2: lane i%8 of each half row, in sa (two masked multiply-adds per lookup)
+//   GSUB 4: lane i%4 of each quad, in sa for I0..I0+3 and sb for I0+4..I0+7
+template <int GSUB, int I0>
+__device__ __forceinline__ void lookup8(float (&acc)[kBatch], uint32_t w0, uint32_t w1, uint32_t lane_off,
+                                        float sa, float sb)
 {
-    int ab = __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, a), CTRL, 0xf, BANKS, BANKS == 0xf);
-    return __builtin_fmaf(__builtin_bit_cast(float, ab), v, acc);
-}
-
-constexpr int kRowBcast = 0x150;  // DPP control of row_newbcast:0
-
-// acc += scale(output I, slot BO) * v, the scale coming from the lane that holds it.
-//   GSUB 1: lane I%16 of the row, register slot I/16
-//   GSUB 2: lane I%8 of each half row (two masked instructions), slot I/8
-//   GSUB 4: lane I%4 of each quad, slot I/4
-template <int GSUB, int QO, int I, int BO, int NSC>
-__device__ __forceinline__ float scaled_add(const float (&sc)[NSC], float v, float acc)
-{
-    if constexpr (GSUB == 1) {
-        return fma_bcast<kRowBcast + (I % 16), 0xf>(sc[(I / 16) * QO + BO], v, acc);
+    uint32_t tmp[8];
+    if constexpr (GSUB == 1 && (I0 % 16) == 0) {
+        asm volatile(LG_ADDR_AND_READ
+                     LG_WAIT(7) LG_FMA(0, 23, 8, LG_ROW(0)) LG_WAIT(6) LG_FMA(1, 23, 9, LG_ROW(1))
+                     LG_WAIT(5) LG_FMA(2, 23, 10, LG_ROW(2)) LG_WAIT(4) LG_FMA(3, 23, 11, LG_ROW(3))
+                     LG_WAIT(3) LG_FMA(4, 23, 12, LG_ROW(4)) LG_WAIT(2) LG_FMA(5, 23, 13, LG_ROW(5))
+                     LG_WAIT(1) LG_FMA(6, 23, 14, LG_ROW(6)) LG_WAIT(0) LG_FMA(7, 23, 15, LG_ROW(7))
+                     : LG_OUT(acc, I0, tmp)
+                     : LG_IN(w0, w1, lane_off), "v"(sa)
+                     : "memory");
+    } else if constexpr (GSUB == 1) {
+        asm volatile(LG_ADDR_AND_READ
+                     LG_WAIT(7) LG_FMA(0, 23, 8, LG_ROW(8)) LG_WAIT(6) LG_FMA(1, 23, 9, LG_ROW(9))
+                     LG_WAIT(5) LG_FMA(2, 23, 10, LG_ROW(10)) LG_WAIT(4) LG_FMA(3, 23, 11, LG_ROW(11))
+                     LG_WAIT(3) LG_FMA(4, 23, 12, LG_ROW(12)) LG_WAIT(2) LG_FMA(5, 23, 13, LG_ROW(13))
+                     LG_WAIT(1) LG_FMA(6, 23, 14, LG_ROW(14)) LG_WAIT(0) LG_FMA(7, 23, 15, LG_ROW(15))
+                     : LG_OUT(acc, I0, tmp)
+                     : LG_IN(w0, w1, lane_off), "v"(sa)
+                     : "memory");
     } else if constexpr (GSUB == 2) {
-        const float s = sc[(I / 8) * QO + BO];
-        acc = fma_bcast<kRowBcast + (I % 8), 0x3>(s, v, acc);
-        return fma_bcast<kRowBcast + 8 + (I % 8), 0xc>(s, v, acc);
+        asm volatile(LG_ADDR_AND_READ
+                     LG_WAIT(7) LG_FMA(0, 23, 8, LG_LOHALF(0)) LG_FMA(0, 23, 8, LG_HIHALF(8))
+                     LG_WAIT(6) LG_FMA(1, 23, 9, LG_LOHALF(1)) LG_FMA(1, 23, 9, LG_HIHALF(9))
+                     LG_WAIT(5) LG_FMA(2, 23, 10, LG_LOHALF(2)) LG_FMA(2, 23, 10, LG_HIHALF(10))
+                     LG_WAIT(4) LG_FMA(3, 23, 11, LG_LOHALF(3)) LG_FMA(3, 23, 11, LG_HIHALF(11))
+                     LG_WAIT(3) LG_FMA(4, 23, 12, LG_LOHALF(4)) LG_FMA(4, 23, 12, LG_HIHALF(12))
+                     LG_WAIT(2) LG_FMA(5, 23, 13, LG_LOHALF(5)) LG_FMA(5, 23, 13, LG_HIHALF(13))
+                     LG_WAIT(1) LG_FMA(6, 23, 14, LG_LOHALF(6)) LG_FMA(6, 23, 14, LG_HIHALF(14))
+                     LG_WAIT(0) LG_FMA(7, 23, 15, LG_LOHALF(7)) LG_FMA(7, 23, 15, LG_HIHALF(15))
+                     : LG_OUT(acc, I0, tmp)
+                     : LG_IN(w0, w1, lane_off), "v"(sa)
+                     : "memory");
     } else {
-        return fma_bcast<(I % 4) * 0x55, 0xf>(sc[(I / 4) * QO + BO], v, acc);
+        asm volatile(LG_ADDR_AND_READ
+                     LG_WAIT(7) LG_FMA(0, 23, 8, LG_QUAD(0)) LG_WAIT(6) LG_FMA(1, 23, 9, LG_QUAD(1))
+                     LG_WAIT(5) LG_FMA(2, 23, 10, LG_QUAD(2)) LG_WAIT(4) LG_FMA(3, 23, 11, LG_QUAD(3))
+                     LG_WAIT(3) LG_FMA(4, 24, 12, LG_QUAD(0)) LG_WAIT(2) LG_FMA(5, 24, 13, LG_QUAD(1))
+                     LG_WAIT(1) LG_FMA(6, 24, 14, LG_QUAD(2)) LG_WAIT(0) LG_FMA(7, 24, 15, LG_QUAD(3))
+                     : LG_OUT(acc, I0, tmp)
+                     : LG_IN(w0, w1, lane_off), "v"(sa), "v"(sb)
+                     : "memory");
+    }
+}
+
+// acc[I0..I0+7] += offset scale (fetched across lanes like any scale) * v, no table involved.
+// Operands: %0-%7 accumulators, %8 v, %9 (%10) scale registers.
+#define LG_OFMA(k, S, CTRL) "v_fmac_f32_dpp %" #k ", %" #S ", %8" CTRL
+#define LG_OOUT(acc, I0)                                                                           \
+    "+v"(acc[I0 + 0]), "+v"(acc[I0 + 1]), "+v"(acc[I0 + 2]), "+v"(acc[I0 + 3]), "+v"(acc[I0 + 4]),   \
+        "+v"(acc[I0 + 5]), "+v"(acc[I0 + 6]), "+v"(acc[I0 + 7])
+template <int GSUB, int I0>
+__device__ __forceinline__ void offset8(float (&acc)[kBatch], float v, float sa, float sb)
+{
+    if constexpr (GSUB == 1 && (I0 % 16) == 0) {
+        asm volatile("s_nop 1\n" LG_OFMA(0, 9, LG_ROW(0)) LG_OFMA(1, 9, LG_ROW(1)) LG_OFMA(2, 9, LG_ROW(2))
+                     LG_OFMA(3, 9, LG_ROW(3)) LG_OFMA(4, 9, LG_ROW(4)) LG_OFMA(5, 9, LG_ROW(5))
+                     LG_OFMA(6, 9, LG_ROW(6)) LG_OFMA(7, 9, LG_ROW(7))
+                     : LG_OOUT(acc, I0) : "v"(v), "v"(sa));
+    } else if constexpr (GSUB == 1) {
+        asm volatile("s_nop 1\n" LG_OFMA(0, 9, LG_ROW(8)) LG_OFMA(1, 9, LG_ROW(9)) LG_OFMA(2, 9, LG_ROW(10))
+                     LG_OFMA(3, 9, LG_ROW(11)) LG_OFMA(4, 9, LG_ROW(12)) LG_OFMA(5, 9, LG_ROW(13))
+                     LG_OFMA(6, 9, LG_ROW(14)) LG_OFMA(7, 9, LG_ROW(15))
+                     : LG_OOUT(acc, I0) : "v"(v), "v"(sa));
+    } else if constexpr (GSUB == 2) {
+        asm volatile("s_nop 1\n" LG_OFMA(0, 9, LG_LOHALF(0)) LG_OFMA(0, 9, LG_HIHALF(8))
+                     LG_OFMA(1, 9, LG_LOHALF(1)) LG_OFMA(1, 9, LG_HIHALF(9))
+                     LG_OFMA(2, 9, LG_LOHALF(2)) LG_OFMA(2, 9, LG_HIHALF(10))
+                     LG_OFMA(3, 9, LG_LOHALF(3)) LG_OFMA(3, 9, LG_HIHALF(11))
+                     LG_OFMA(4, 9, LG_LOHALF(4)) LG_OFMA(4, 9, LG_HIHALF(12))
+                     LG_OFMA(5, 9, LG_LOHALF(5)) LG_OFMA(5, 9, LG_HIHALF(13))
+                     LG_OFMA(6, 9, LG_LOHALF(6)) LG_OFMA(6, 9, LG_HIHALF(14))
+                     LG_OFMA(7, 9, LG_LOHALF(7)) LG_OFMA(7, 9, LG_HIHALF(15))
+                     : LG_OOUT(acc, I0) : "v"(v), "v"(sa));
+    } else {
+        asm volatile("s_nop 1\n" LG_OFMA(0, 9, LG_QUAD(0)) LG_OFMA(1, 9, LG_QUAD(1)) LG_OFMA(2, 9, LG_QUAD(2))
+                     LG_OFMA(3, 9, LG_QUAD(3)) LG_OFMA(4, 10, LG_QUAD(0)) LG_OFMA(5, 10, LG_QUAD(1))
+                     LG_OFMA(6, 10, LG_QUAD(2)) LG_OFMA(7, 10, LG_QUAD(3))
+                     : LG_OOUT(acc, I0) : "v"(v), "v"(sa), "v"(sb));
     }
 }
 
@@ -101,6 +196,7 @@ __device__ __forceinline__ void build_quarter(float *col, int qtr, const float (
             top + (((h & 1) ? f[3] : -f[3]) + ((h & 2) ? f[4] : -f[4]) + ((h & 4) ? f[5] : -f[5]));
 #pragma unroll
         for (int t = 0; t < 8; t++) q[(h * 8 + t) * kLanes] = hi + lo[t];
+        __builtin_amdgcn_sched_barrier(0);  // store each row of 8 before computing the next
     }
 }
 
@@ -110,36 +206,62 @@ struct TileRegs {
     uint32_t scale[GSUB * QO];
 };
 
+// Where the next tile's loads of a wavefront come from (all lanes the same dummy line when the
+// workgroup has no next k-block, see tile_address).
+struct NextTile {
+    const u32x4 *sign;    // this lane's first sign vector
+    size_t sign_stride;   // in u32x4 units between units
+    const uint32_t *scale;
+};
+
+// Addresses of tile `tile` for this lane.  `real` is wave-uniform; when false every lane reads
+// the first bytes of the arrays instead (one cached line).  Written with masks rather than
+// conditionals so that no branch appears: with straight-line code the compiler's wait counts
+// for the loads stay exact.
 template <int Q, int QO, int GSUB>
-__device__ __forceinline__ void load_tile(TileRegs<Q, QO, GSUB> &r, const u32x4 *signs,
-                                          const uint32_t *scales, size_t tile, int lane)
+__device__ __forceinline__ NextTile tile_address(const u32x4 *signs, const uint32_t *scales, size_t tile,
+                                                 int lane, bool real)
 {
-    const uint32_t *cp = scales + (tile * kLanes + lane) * (size_t)(GSUB * QO);
-#pragma unroll
-    for (int d = 0; d < GSUB * QO; d++) r.scale[d] = __builtin_nontemporal_load(cp + d);
-    const u32x4 *sp = signs + tile * (size_t)(2 * Q * kLanes) + lane;
-#pragma unroll
-    for (int u = 0; u < 2 * Q; u++) r.sign[u] = __builtin_nontemporal_load(sp + u * kLanes);
+    const size_t m = (size_t)0 - (size_t)real;  // all ones or zero
+    NextTile n;
+    n.scale = scales + (((tile * kLanes + lane) * (size_t)(GSUB * QO)) & m);
+    n.sign = signs + ((tile * (size_t)(2 * Q * kLanes) + lane) & m);
+    n.sign_stride = (size_t)kLanes & m;
+    return n;
 }
 
-// This lane's 8 activations of k-block ts as fp32 (zero beyond k).
-__device__ __forceinline__ void load_activations(const __half *x, int x_stride, int k, int ts, int lane,
-                                                 float (&f)[8])
+template <int Q, int QO, int GSUB>
+__device__ __forceinline__ void load_tile(TileRegs<Q, QO, GSUB> &r, const NextTile &n)
+{
+#pragma unroll
+    for (int d = 0; d < GSUB * QO; d++) r.scale[d] = __builtin_nontemporal_load(n.scale + d);
+#pragma unroll
+    for (int u = 0; u < 2 * Q; u++) r.sign[u] = __builtin_nontemporal_load(n.sign + u * n.sign_stride);
+}
+
+// Raw fp16 activations of this lane's chunk in k-block ts (zero beyond k or when !valid).
+// Branch free for the same reason.  x is contiguous.
+__device__ __forceinline__ u32x4 load_activations(const __half *x, int k, int ts, int lane, bool valid)
 {
     const int kpos = (ts * kLanes + lane) * kChunk;
-    if (kpos < k) {
-        if (x_stride == 1) {
-            const uint4 raw = *reinterpret_cast<const uint4 *>(x + kpos);
-            const __half *hp = reinterpret_cast<const __half *>(&raw);
+    const uint32_t m = 0u - (uint32_t)(valid && kpos < k);
+    const u32x4 raw = *reinterpret_cast<const u32x4 *>(x + (kpos & (int)m));
+    u32x4 out = raw;
+    out.x &= m;
+    out.y &= m;
+    out.z &= m;
+    out.w &= m;
+    return out;
+}
+
+__device__ __forceinline__ void unpack_activations(const u32x4 &raw, float (&f)[8])
+{
+    const uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
 #pragma unroll
-            for (int j = 0; j < 8; j++) f[j] = __half2float(hp[j]);
-        } else {
-#pragma unroll
-            for (int j = 0; j < 8; j++) f[j] = __half2float(x[(size_t)(kpos + j) * x_stride]);
-        }
-    } else {
-#pragma unroll
-        for (int j = 0; j < 8; j++) f[j] = 0.f;
+    for (int j = 0; j < 4; j++) {
+        const __half2 h2 = *reinterpret_cast<const __half2 *>(&w[j]);
+        f[2 * j] = __low2float(h2);
+        f[2 * j + 1] = __high2float(h2);
     }
 }
 
@@ -154,14 +276,19 @@ __device__ __forceinline__ void build_tables(float *table, const float (&f)[8], 
     __syncthreads();
 }
 
-// All lookups of one tile (32 outputs x Q planes for this lane's chunk) into acc.
+// All lookups of one tile (32 outputs x Q planes for this lane's chunk) into acc, and the
+// refill of the same registers with the next tile: each 16-byte sign vector is reloaded right
+// after its 16 lookups, the scale words right after their conversion.  The loads of a
+// wavefront are thereby spread evenly over its compute instead of being issued in a burst
+// (vector memory issue blocks the wavefront while the request queue of the CU is full).
+// Scale register of output i, plane/offset slot bo: sc[(i / (16/GSUB)) * QO + bo].
 template <int Q, bool OFF, int GSUB>
-__device__ __forceinline__ void process_tile(const TileRegs<Q, Q + (OFF ? 1 : 0), GSUB> &t,
-                                             const float *table, uint32_t lane_off, float chunk_sum,
-                                             float (&acc)[kBatch])
+__device__ __forceinline__ void process_tile(TileRegs<Q, Q + (OFF ? 1 : 0), GSUB> &t, uint32_t lane_off,
+                                             float chunk_sum, float (&acc)[kBatch], const NextTile &next)
 {
     constexpr int QO = Q + (OFF ? 1 : 0);
     constexpr int NSC = 2 * GSUB * QO;  // scales held per lane
+    constexpr int SUBL = 16 / GSUB;     // outputs per scale slot
     float sc[NSC];
 #pragma unroll
     for (int d = 0; d < GSUB * QO; d++) {
@@ -169,30 +296,83 @@ __device__ __forceinline__ void process_tile(const TileRegs<Q, Q + (OFF ? 1 : 0)
         sc[2 * d] = __low2float(h2);
         sc[2 * d + 1] = __high2float(h2);
     }
+#pragma unroll
+    for (int d = 0; d < GSUB * QO; d++) t.scale[d] = __builtin_nontemporal_load(next.scale + d);
+    // scale registers of the 8 outputs starting at I0 (second one only differs for GSUB 4)
+    auto sa = [&](auto I0, int bo) { return sc[(I0 / SUBL) * QO + bo]; };
+    auto sb = [&](auto I0, int bo) { return sc[((I0 + 4) / SUBL) * QO + bo]; };
 
     // offset term: q_bias[group][out] * (sum of this lane's 8 activations)
     if constexpr (OFF) {
-        static_for<kBatch>([&](auto I) {
-            acc[I] = scaled_add<GSUB, QO, I, Q, NSC>(sc, chunk_sum, acc[I]);
+        static_for<4>([&](auto G) {
+            constexpr int I0 = G * 8;
+            offset8<GSUB, I0>(acc, chunk_sum, sa(std::integral_constant<int, I0>{}, Q),
+                              sb(std::integral_constant<int, I0>{}, Q));
         });
     }
 
     static_for<2 * Q>([&](auto U) {
+        // one unit = 16 lookups = one 16-byte sign vector (plane b, output half h)
         constexpr int b = U / 2, h = U % 2;
+        constexpr int I0 = h * 16;
         const u32x4 w4 = t.sign[U];
-        const uint32_t w[4] = {w4.x, w4.y, w4.z, w4.w};
-        static_for<16>([&](auto P) {
-            constexpr int i = h * 16 + P;
-            // address = entry * 256 + lane * 4: sign byte -> address byte 1,
-            // lane_off -> address byte 0, upper bytes zero
-            constexpr uint32_t sel = 0x0c0c0400u | ((uint32_t)(P % 4) << 8);
-            const uint32_t addr = __builtin_amdgcn_perm(w[P / 4], lane_off, sel);
-            const float v = lds_lookup(table, addr);
-            acc[i] = scaled_add<GSUB, QO, i, b, NSC>(sc, v, acc[i]);
-        });
-        // keep the 16 lookups of a unit together: bounds the registers in flight
-        __builtin_amdgcn_sched_barrier(0);
+        lookup8<GSUB, I0>(acc, w4.x, w4.y, lane_off, sa(std::integral_constant<int, I0>{}, b),
+                          sb(std::integral_constant<int, I0>{}, b));
+        lookup8<GSUB, I0 + 8>(acc, w4.z, w4.w, lane_off, sa(std::integral_constant<int, I0 + 8>{}, b),
+                              sb(std::integral_constant<int, I0 + 8>{}, b));
+        t.sign[U] = __builtin_nontemporal_load(next.sign + U * next.sign_stride);
     });
+}
+
+// Sum of each of the 32 accumulators over the 64 lanes, VALU only, fixed order.
+// Halving butterfly: each step pairs accumulators (i, i+half) and leaves in every lane the one
+// its lane bit selects, summed with the partner lane's copy.  Lane bit 5 / 4 steps use the
+// gfx950 half-wave / row swaps, bits 3 and 2 use masked row shifts, bits 1 and 0 quad
+// permutes.  Lane L ends with the total of output L >> 1 (both lanes of a pair hold it).
+__device__ __forceinline__ float reduce_across_lanes(float (&acc)[kBatch], int lane)
+{
+    auto as_u = [](float v) { return __builtin_bit_cast(unsigned, v); };
+    auto as_f = [](unsigned v) { return __builtin_bit_cast(float, v); };
+    // lane bit 5: swap the upper half of A with the lower half of B, then add
+    static_for<16>([&](auto I) {
+        const auto r = __builtin_amdgcn_permlane32_swap(as_u(acc[I]), as_u(acc[I + 16]), false, false);
+        acc[I] = as_f(r[0]) + as_f(r[1]);
+    });
+    // lane bit 4: swap the odd rows of A with the even rows of B, then add
+    static_for<8>([&](auto I) {
+        const auto r = __builtin_amdgcn_permlane16_swap(as_u(acc[I]), as_u(acc[I + 8]), false, false);
+        acc[I] = as_f(r[0]) + as_f(r[1]);
+    });
+    // lane bit 3: banks 0,1 (lanes 0..7 of a row) keep A and fetch A from lane+8,
+    //             banks 2,3 keep B and fetch B from lane-8
+    static_for<4>([&](auto I) {
+        const float a = acc[I], b = acc[I + 4];
+        const unsigned got = __builtin_amdgcn_update_dpp(
+            __builtin_amdgcn_update_dpp(0u, as_u(a), 0x108 /* row_shl:8 */, 0xf, 0x3, false), as_u(b),
+            0x118 /* row_shr:8 */, 0xf, 0xc, false);
+        acc[I] = ((lane & 8) ? b : a) + as_f(got);
+    });
+    // lane bit 2: banks 0,2 keep A (fetch from lane+4), banks 1,3 keep B (fetch from lane-4)
+    static_for<2>([&](auto I) {
+        const float a = acc[I], b = acc[I + 2];
+        const unsigned got = __builtin_amdgcn_update_dpp(
+            __builtin_amdgcn_update_dpp(0u, as_u(a), 0x104 /* row_shl:4 */, 0xf, 0x5, false), as_u(b),
+            0x114 /* row_shr:4 */, 0xf, 0xa, false);
+        acc[I] = ((lane & 4) ? b : a) + as_f(got);
+    });
+    // lane bit 1: exchange inside quads (lane ^ 2)
+    {
+        const float a = acc[0], b = acc[1];
+        const bool up = (lane & 2) != 0;
+        const float send = up ? a : b;
+        const unsigned got = __builtin_amdgcn_update_dpp(0u, as_u(send), 0x4e /* quad_perm:[2,3,0,1] */, 0xf,
+                                                         0xf, true);
+        acc[0] = (up ? b : a) + as_f(got);
+    }
+    // lane bit 0: both lanes of a pair end with the same total
+    const unsigned other =
+        __builtin_amdgcn_update_dpp(0u, as_u(acc[0]), 0xb1 /* quad_perm:[1,0,3,2] */, 0xf, 0xf, true);
+    return acc[0] + as_f(other);
 }
 
 template <int Q, bool OFF, int GSUB>
@@ -200,7 +380,6 @@ __global__ __launch_bounds__(768) void lut_matvec_kernel(MatvecArgs a)
 {
     constexpr int QO = Q + (OFF ? 1 : 0);
     __shared__ float table[kTableFloats];
-    __shared__ int last_flag;
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -221,44 +400,30 @@ __global__ __launch_bounds__(768) void lut_matvec_kernel(MatvecArgs a)
 #pragma unroll
     for (int i = 0; i < kBatch; i++) acc[i] = 0.f;
 
-    // byte 0 of every lookup address: this lane's column
-    const uint32_t lane_off = (uint32_t)lane * 4u;
-    // inactive wavefronts (beyond the last batch) stream batch 0 and discard the result
+    // Bytes 0, 2 and 3 of every lookup address: this lane's column plus the LDS address of the
+    // table (a multiple of 64 KiB, in fact 0: the table is the kernel's only LDS object).
+    const uint32_t lane_off =
+        (uint32_t)lane * 4u + (uint32_t)(size_t)(__attribute__((address_space(3))) float *)table;
+    // wavefronts beyond the last batch stream batch 0 and discard the result
     const size_t tile0 = (size_t)(active ? nb : 0) * a.ts;
 
-    TileRegs<Q, QO, GSUB> cur, nxt;
-    load_tile(cur, signs, scales, tile0 + ts0, lane);
+    // One tile of registers per wavefront, refilled in place while it is consumed.
+    TileRegs<Q, QO, GSUB> tile;
+    u32x4 xraw = load_activations(x, a.k, ts0, lane, true);
+    load_tile(tile, tile_address<Q, QO, GSUB>(signs, scales, tile0 + ts0, lane, true));
 
-    float f[8];
-    for (int ts = ts0; ts < ts1 - 1; ts++) {
-        load_activations(x, a.x_stride, a.k, ts, lane, f);
-        build_tables(table, f, lane, wave, waves);
-        load_tile(nxt, signs, scales, tile0 + ts + 1, lane);
-        const float chunk_sum = ((f[0] + f[1]) + (f[2] + f[3])) + ((f[4] + f[5]) + (f[6] + f[7]));
-        process_tile<Q, OFF, GSUB>(cur, table, lane_off, chunk_sum, acc);
-        cur = nxt;
-    }
-    {
-        load_activations(x, a.x_stride, a.k, ts1 - 1, lane, f);
+    for (int ts = ts0; ts < ts1; ts++) {
+        float f[8];
+        unpack_activations(xraw, f);
+        const bool more = ts + 1 < ts1;
+        xraw = load_activations(x, a.k, ts + 1, lane, more);
         build_tables(table, f, lane, wave, waves);
         const float chunk_sum = ((f[0] + f[1]) + (f[2] + f[3])) + ((f[4] + f[5]) + (f[6] + f[7]));
-        process_tile<Q, OFF, GSUB>(cur, table, lane_off, chunk_sum, acc);
+        process_tile<Q, OFF, GSUB>(tile, lane_off, chunk_sum, acc,
+                                   tile_address<Q, QO, GSUB>(signs, scales, tile0 + ts + 1, lane, more));
     }
 
-    // Reduce the 64 per-lane partials of each of the 32 outputs.  Halving butterfly over lane
-    // bits 5..1 (after the step with mask M, value index bit log2(M)-1 equals the lane's bit
-    // log2(M)), then one full exchange over bit 0: lane L ends with the total of output L>>1.
-    static_for<5>([&](auto LV) {
-        constexpr int half = 16 >> LV;
-        constexpr int mask = half * 2;
-        const bool upper = (lane & mask) != 0;
-        static_for<half>([&](auto I) {
-            const float keep = upper ? acc[I + half] : acc[I];
-            const float send = upper ? acc[I] : acc[I + half];
-            acc[I] = keep + __shfl_xor(send, mask, 64);
-        });
-    });
-    const float total = acc[0] + __shfl_xor(acc[0], 1, 64);
+    const float total = reduce_across_lanes(acc, lane);
 
     const int out = nb * kBatch + (lane >> 1);
     __half *y = reinterpret_cast<__half *>(a.y);
@@ -271,16 +436,19 @@ __global__ __launch_bounds__(768) void lut_matvec_kernel(MatvecArgs a)
     // all of them in ascending split order.
     const size_t npad = (size_t)a.nb * kBatch;
     if (active && (lane & 1) == 0) a.partials[(size_t)ks * npad + out] = total;
-    __threadfence();
-    __syncthreads();
+    __syncthreads();  // every wavefront's partial stores have completed (workgroup scope)
     if (tid == 0) {
+        // One device-scope release for the whole workgroup (the barrier orders the other
+        // wavefronts' stores before it), then the arrival ticket; the last arrival acquires.
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
         const unsigned ticket =
-            __hip_atomic_fetch_add(a.counters + ntile, 1u, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
-        last_flag = (ticket == (unsigned)(a.k_splits - 1));
+            __hip_atomic_fetch_add(a.counters + ntile, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        const int last = (ticket == (unsigned)(a.k_splits - 1));
+        if (last) __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+        table[0] = last ? 1.f : 0.f;  // the table is dead by now; reuse it as the broadcast slot
     }
     __syncthreads();
-    if (!last_flag) return;
-    __threadfence();
+    if (table[0] == 0.f) return;
     for (int o = tid; o < waves * kBatch; o += blockDim.x) {
         const int col = ntile * waves * kBatch + o;
         if (col < a.n) {
