@@ -177,23 +177,24 @@ __device__ __forceinline__ void offset8(float (&acc)[kBatch], float v, float sa,
     }
 }
 
-// Build one quarter (entries qtr*64 .. qtr*64+63, qtr wave-uniform) of this lane's 256-entry
+// Build one eighth (entries part*32 .. part*32+31, part wave-uniform) of this lane's 256-entry
 // table from its 8 activations f[0..7]:  entry(idx) = sum_j (bit_j(idx) ? +f[j] : -f[j]).
-// Split as (bits 6,7 fixed by qtr) + (bits 3..5) + (bits 0..2) so no entry is more than a
-// few fp32 additions away from the inputs.  One code path for all quarters: only `top` and
-// the base address depend on qtr.
-__device__ __forceinline__ void build_quarter(float *col, int qtr, const float (&f)[8])
+// Split as (bits 5..7 fixed by part) + (bits 3,4) + (bits 0..2) so no entry is more than a few
+// fp32 additions away from the inputs.  One code path for all parts: only `top` and the base
+// address depend on part.
+constexpr int kBuildParts = 8;
+__device__ __forceinline__ void build_part(float *col, int part, const float (&f)[8])
 {
     float lo[8];
 #pragma unroll
     for (int t = 0; t < 8; t++)
         lo[t] = ((t & 1) ? f[0] : -f[0]) + ((t & 2) ? f[1] : -f[1]) + ((t & 4) ? f[2] : -f[2]);
-    const float top = ((qtr & 1) ? f[6] : -f[6]) + ((qtr & 2) ? f[7] : -f[7]);
-    float *q = col + qtr * (64 * kLanes);
+    const float top =
+        (((part & 1) ? f[5] : -f[5]) + ((part & 2) ? f[6] : -f[6])) + ((part & 4) ? f[7] : -f[7]);
+    float *q = col + part * (32 * kLanes);
 #pragma unroll
-    for (int h = 0; h < 8; h++) {
-        const float hi =
-            top + (((h & 1) ? f[3] : -f[3]) + ((h & 2) ? f[4] : -f[4]) + ((h & 4) ? f[5] : -f[5]));
+    for (int h = 0; h < 4; h++) {
+        const float hi = top + (((h & 1) ? f[3] : -f[3]) + ((h & 2) ? f[4] : -f[4]));
 #pragma unroll
         for (int t = 0; t < 8; t++) q[(h * 8 + t) * kLanes] = hi + lo[t];
         __builtin_amdgcn_sched_barrier(0);  // store each row of 8 before computing the next
@@ -263,17 +264,20 @@ __device__ __forceinline__ void unpack_activations(const u32x4 &raw, float (&f)[
         f[2 * j] = __low2float(h2);
         f[2 * j + 1] = __high2float(h2);
     }
+    // Pin the conversion here for every wavefront.  Only some wavefronts build table parts; left
+    // alone, the compiler sinks the activation load itself into that branch, behind all the tile
+    // loads, and then has to wait for every outstanding load before the first build.
+#pragma unroll
+    for (int j = 0; j < 8; j++) asm volatile("" : "+v"(f[j]));
 }
 
-// Rebuild the table set for this lane's chunk.  Two barriers: the first makes sure every
-// lookup into the previous table set has completed, the second publishes the new one.
+// This wavefront's share of the table set of one k-block: eight parts spread over the
+// wavefronts of the workgroup.  No barrier here; the caller synchronises.
 __device__ __forceinline__ void build_tables(float *table, const float (&f)[8], int lane, int wave,
                                              int waves)
 {
-    __syncthreads();
     float *col = table + lane;
-    for (int task = wave; task < 4; task += waves) build_quarter(col, task, f);
-    __syncthreads();
+    for (int task = wave; task < kBuildParts; task += waves) build_part(col, task, f);
 }
 
 // All lookups of one tile (32 outputs x Q planes for this lane's chunk) into acc, and the
@@ -379,7 +383,8 @@ template <int Q, bool OFF, int GSUB>
 __global__ __launch_bounds__(768) void lut_matvec_kernel(MatvecArgs a)
 {
     constexpr int QO = Q + (OFF ? 1 : 0);
-    __shared__ float table[kTableFloats];
+    // Two table sets: while the lookups of k-block t read one, the other is rebuilt for t+1.
+    __shared__ float table[2 * kTableFloats];
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -401,26 +406,36 @@ __global__ __launch_bounds__(768) void lut_matvec_kernel(MatvecArgs a)
     for (int i = 0; i < kBatch; i++) acc[i] = 0.f;
 
     // Bytes 0, 2 and 3 of every lookup address: this lane's column plus the LDS address of the
-    // table (a multiple of 64 KiB, in fact 0: the table is the kernel's only LDS object).
-    const uint32_t lane_off =
+    // table set in use (a multiple of 64 KiB: the tables are the kernel's only LDS object).
+    const uint32_t lane_base =
         (uint32_t)lane * 4u + (uint32_t)(size_t)(__attribute__((address_space(3))) float *)table;
     // wavefronts beyond the last batch stream batch 0 and discard the result
     const size_t tile0 = (size_t)(active ? nb : 0) * a.ts;
 
-    // One tile of registers per wavefront, refilled in place while it is consumed.
+    // One tile of registers per wavefront, refilled in place while it is consumed; activations
+    // are fetched two k-blocks ahead because the table of k-block t+1 is built during t.
     TileRegs<Q, QO, GSUB> tile;
-    u32x4 xraw = load_activations(x, a.k, ts0, lane, true);
+    u32x4 xcur = load_activations(x, a.k, ts0, lane, true);
+    u32x4 xnext = load_activations(x, a.k, ts0 + 1, lane, ts0 + 1 < ts1);
     load_tile(tile, tile_address<Q, QO, GSUB>(signs, scales, tile0 + ts0, lane, true));
 
+    float f[8];
+    unpack_activations(xcur, f);
+    build_tables(table, f, lane, wave, waves);
+    __syncthreads();
+
     for (int ts = ts0; ts < ts1; ts++) {
-        float f[8];
-        unpack_activations(xraw, f);
-        const bool more = ts + 1 < ts1;
-        xraw = load_activations(x, a.k, ts + 1, lane, more);
-        build_tables(table, f, lane, wave, waves);
+        const int cur = (ts - ts0) & 1;
         const float chunk_sum = ((f[0] + f[1]) + (f[2] + f[3])) + ((f[4] + f[5]) + (f[6] + f[7]));
-        process_tile<Q, OFF, GSUB>(tile, lane_off, chunk_sum, acc,
+        const bool more = ts + 1 < ts1;
+        // table set of the next k-block (all zero activations past the end: harmless, unused)
+        unpack_activations(xnext, f);
+        xnext = load_activations(x, a.k, ts + 2, lane, ts + 2 < ts1);
+        build_tables(table + (cur ^ 1) * kTableFloats, f, lane, wave, waves);
+        process_tile<Q, OFF, GSUB>(tile, lane_base + (uint32_t)cur * (kTableFloats * 4u), chunk_sum, acc,
                                    tile_address<Q, QO, GSUB>(signs, scales, tile0 + ts + 1, lane, more));
+        // the next table set is complete and every lookup into the current one has finished
+        __syncthreads();
     }
 
     const float total = reduce_across_lanes(acc, lane);
@@ -432,20 +447,21 @@ __global__ __launch_bounds__(768) void lut_matvec_kernel(MatvecArgs a)
         return;
     }
 
-    // split-k: publish this workgroup's partials, the last workgroup of the column tile adds
-    // all of them in ascending split order.
+    // split-k: publish this workgroup's partials; the last workgroup of the column tile to
+    // arrive adds all of them in ascending split order.  Partials and the arrival ticket are
+    // device-scope atomic accesses (written through to / read from the coherence point), so no
+    // cache write-back or invalidate is needed; each wavefront waits for its own stores to
+    // complete before the barrier, and the ticket is taken after the barrier.
     const size_t npad = (size_t)a.nb * kBatch;
-    if (active && (lane & 1) == 0) a.partials[(size_t)ks * npad + out] = total;
-    __syncthreads();  // every wavefront's partial stores have completed (workgroup scope)
+    if (active && (lane & 1) == 0)
+        __hip_atomic_store(a.partials + (size_t)ks * npad + out, total, __ATOMIC_RELAXED,
+                           __HIP_MEMORY_SCOPE_AGENT);
+    __builtin_amdgcn_s_waitcnt(0);  // vmcnt(0): this wavefront's partial stores are complete
+    __syncthreads();
     if (tid == 0) {
-        // One device-scope release for the whole workgroup (the barrier orders the other
-        // wavefronts' stores before it), then the arrival ticket; the last arrival acquires.
-        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
         const unsigned ticket =
             __hip_atomic_fetch_add(a.counters + ntile, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        const int last = (ticket == (unsigned)(a.k_splits - 1));
-        if (last) __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
-        table[0] = last ? 1.f : 0.f;  // the table is dead by now; reuse it as the broadcast slot
+        table[0] = (ticket == (unsigned)(a.k_splits - 1)) ? 1.f : 0.f;  // the tables are dead by now
     }
     __syncthreads();
     if (table[0] == 0.f) return;
@@ -454,7 +470,8 @@ __global__ __launch_bounds__(768) void lut_matvec_kernel(MatvecArgs a)
         if (col < a.n) {
             float s = 0.f;
             for (int i = 0; i < a.k_splits; i++)
-                s += __builtin_nontemporal_load(a.partials + (size_t)i * npad + col);
+                s += __hip_atomic_load(a.partials + (size_t)i * npad + col, __ATOMIC_RELAXED,
+                                       __HIP_MEMORY_SCOPE_AGENT);
             y[(size_t)col * a.y_stride] = __float2half_rn(s);
         }
     }
