@@ -36,6 +36,7 @@ int hip_fail(hipError_t e, const char *what)
 }
 
 constexpr int kMaxWaves = 12;  // the kernel is compiled for at most 768 threads per workgroup
+constexpr int kMaxSplits = 128;  // the split-k arrival count has 8 bits and the sum 2^56 / 2^48 addends
 
 struct Plan {
     int waves;             // wavefronts (= output batches) per workgroup
@@ -52,9 +53,8 @@ struct lutgemm_weight {
     int compute_units;
     uint8_t *d_signs;
     uint16_t *d_scales;
-    float *d_partials;
-    unsigned *d_counters;
-    size_t partial_bytes, counter_bytes;
+    unsigned long long *d_accum;  // split-k accumulators, one 64-bit word per (padded) output
+    size_t accum_bytes;
     Plan plan;
 };
 
@@ -74,7 +74,7 @@ Plan choose_plan(const Shape &s, int cus)
     for (int waves = 1; waves <= kMaxWaves; waves++) {
         const int ntiles = div_up(s.nb, waves);
         const double per_simd = (double)div_up(waves, 4);
-        for (int splits = 1; splits <= s.ts; splits++) {
+        for (int splits = 1; splits <= s.ts && splits <= kMaxSplits; splits++) {
             const int bps = div_up(s.ts, splits);
             const int ks = div_up(s.ts, bps);
             if (ks != splits) continue;  // same plan as a smaller `splits`
@@ -82,7 +82,7 @@ Plan choose_plan(const Shape &s, int cus)
             const double rounds = (double)((wgs + cus - 1) / cus);
             const double build = 160.0 + 40.0;  // quarter build + barriers
             double wg_cost = bps * (build + per_simd * lookup) + per_simd * 180.0;
-            if (ks > 1) wg_cost += 300.0;  // fence + ticket + partial traffic
+            if (ks > 1) wg_cost += 150.0;  // split-k atomic round trip
             // padding waste: wavefronts beyond the last batch still stream a tile
             const double cost = rounds * wg_cost;
             if (cost < best_cost - 1e-9) {
@@ -96,18 +96,12 @@ Plan choose_plan(const Shape &s, int cus)
 
 int alloc_workspace(lutgemm_weight *w)
 {
-    if (w->d_partials) (void)hipFree(w->d_partials);
-    if (w->d_counters) (void)hipFree(w->d_counters);
-    w->d_partials = nullptr;
-    w->d_counters = nullptr;
-    w->partial_bytes = (size_t)w->plan.k_splits * w->shape.nb * kBatch * sizeof(float);
-    w->counter_bytes = (size_t)w->plan.ntiles * sizeof(unsigned);
-    hipError_t e = hipMalloc((void **)&w->d_partials, w->partial_bytes);
-    if (e != hipSuccess) return hip_fail(e, "hipMalloc(partials)");
-    e = hipMalloc((void **)&w->d_counters, w->counter_bytes);
-    if (e != hipSuccess) return hip_fail(e, "hipMalloc(counters)");
-    e = hipMemset(w->d_counters, 0, w->counter_bytes);
-    if (e != hipSuccess) return hip_fail(e, "hipMemset(counters)");
+    if (w->d_accum) return LUTGEMM_OK;  // size depends on the shape only
+    w->accum_bytes = (size_t)w->shape.nb * kBatch * sizeof(unsigned long long);
+    hipError_t e = hipMalloc((void **)&w->d_accum, w->accum_bytes);
+    if (e != hipSuccess) return hip_fail(e, "hipMalloc(split-k accumulators)");
+    e = hipMemset(w->d_accum, 0, w->accum_bytes);
+    if (e != hipSuccess) return hip_fail(e, "hipMemset(split-k accumulators)");
     return LUTGEMM_OK;
 }
 
@@ -186,8 +180,7 @@ int run_matvec(const lutgemm_weight *w, const void *x, void *y, int m, void *str
     lutgemm_kernels::MatvecArgs a{};
     a.signs = w->d_signs;
     a.scales = w->d_scales;
-    a.partials = w->d_partials;
-    a.counters = w->d_counters;
+    a.accum = w->d_accum;
     a.k = s.k;
     a.n = s.n;
     a.ts = s.ts;
@@ -256,7 +249,7 @@ int lutgemm_weight_destroy(lutgemm_weight *w)
 {
     if (!w) return LUTGEMM_OK;
     int st = LUTGEMM_OK;
-    void *ptrs[4] = {w->d_signs, w->d_scales, w->d_partials, w->d_counters};
+    void *ptrs[3] = {w->d_signs, w->d_scales, w->d_accum};
     for (void *p : ptrs)
         if (p) {
             hipError_t e = hipFree(p);
@@ -279,7 +272,7 @@ int lutgemm_weight_info(const lutgemm_weight *w, lutgemm_weight_info_t *info)
     info->sign_bytes = (size_t)s.k / 8 * s.q * s.n;
     info->scale_bytes = (size_t)s.num_groups * s.q * s.n * 2;
     info->offset_bytes = s.has_offset ? (size_t)s.num_groups * s.n * 2 : 0;
-    info->device_bytes = sign_bytes(s) + scale_bytes(s) + w->partial_bytes + w->counter_bytes;
+    info->device_bytes = sign_bytes(s) + scale_bytes(s) + w->accum_bytes;
     return LUTGEMM_OK;
 }
 
@@ -368,8 +361,9 @@ int lutgemm_weight_set_plan(lutgemm_weight *w, int waves_per_group, int k_splits
         p.ntiles = div_up(s.nb, p.waves);
     }
     if (k_splits != 0) {
-        if (k_splits < 1 || k_splits > s.ts)
-            return fail(LUTGEMM_ERR_BAD_SHAPE, "k_splits=%d outside 1..%d", k_splits, s.ts);
+        if (k_splits < 1 || k_splits > s.ts || k_splits > kMaxSplits)
+            return fail(LUTGEMM_ERR_BAD_SHAPE, "k_splits=%d outside 1..%d", k_splits,
+                        s.ts < kMaxSplits ? s.ts : kMaxSplits);
         p.blocks_per_split = div_up(s.ts, k_splits);
         p.k_splits = div_up(s.ts, p.blocks_per_split);
     }

@@ -13,8 +13,8 @@ struct MatvecArgs {
     const uint16_t *scales; // scale tiles (layout.h)
     const void *x;          // fp16 activations, element i at x[i * x_stride]
     void *y;                // fp16 outputs, element j at y[j * y_stride]
-    float *partials;        // [k_splits][nb*32] fp32, used when k_splits > 1
-    unsigned *counters;     // [ntiles] arrival counters, zero between launches
+    unsigned long long *accum;  // [nb*32] split-k accumulators (count | fixed-point sum), zero
+                                // between launches; used when k_splits > 1
     int k, n;
     int ts, nb;             // k-blocks, output batches
     int ntiles;             // column tiles = ceil(nb / waves)

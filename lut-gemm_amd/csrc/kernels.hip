@@ -15,8 +15,9 @@
 //    broadcast from the lane of the same row that holds it (DPP), accumulating in fp32.
 //  * After the last k-block the 64 per-lane partial sums of each output are reduced across the
 //    wavefront in a fixed order.  With more than one k-split the workgroups of a column tile
-//    write fp32 partials and the last one to finish adds them in ascending split order, so the
-//    result is deterministic and no memset or atomic accumulation of y is needed.
+//    add their partials into a per-output fixed-point integer with one 64-bit atomic; the
+//    last arrival finishes the output.  Integer sums do not depend on arrival order, so the
+//    result is deterministic, and no memset or floating-point atomic on y is needed.
 #include <hip/hip_fp16.h>
 #include <hip/hip_runtime.h>
 
@@ -447,35 +448,27 @@ __global__ __launch_bounds__(768) void lut_matvec_kernel(MatvecArgs a)
         return;
     }
 
-    // split-k: publish this workgroup's partials; the last workgroup of the column tile to
-    // arrive adds all of them in ascending split order.  Partials and the arrival ticket are
-    // device-scope atomic accesses (written through to / read from the coherence point), so no
-    // cache write-back or invalidate is needed; each wavefront waits for its own stores to
-    // complete before the barrier, and the ticket is taken after the barrier.
-    const size_t npad = (size_t)a.nb * kBatch;
-    if (active && (lane & 1) == 0)
-        __hip_atomic_store(a.partials + (size_t)ks * npad + out, total, __ATOMIC_RELAXED,
-                           __HIP_MEMORY_SCOPE_AGENT);
-    __builtin_amdgcn_s_waitcnt(0);  // vmcnt(0): this wavefront's partial stores are complete
-    __syncthreads();
-    if (tid == 0) {
-        const unsigned ticket =
-            __hip_atomic_fetch_add(a.counters + ntile, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        table[0] = (ticket == (unsigned)(a.k_splits - 1)) ? 1.f : 0.f;  // the tables are dead by now
-    }
-    __syncthreads();
-    if (table[0] == 0.f) return;
-    for (int o = tid; o < waves * kBatch; o += blockDim.x) {
-        const int col = ntile * waves * kBatch + o;
-        if (col < a.n) {
-            float s = 0.f;
-            for (int i = 0; i < a.k_splits; i++)
-                s += __hip_atomic_load(a.partials + (size_t)i * npad + col, __ATOMIC_RELAXED,
-                                       __HIP_MEMORY_SCOPE_AGENT);
-            y[(size_t)col * a.y_stride] = __float2half_rn(s);
+    // split-k: one 64-bit atomic add per output, no barrier, no second pass.  The word holds an
+    // arrival count in its top 8 bits and the running sum below it, as a biased fixed-point
+    // integer (2^-24 units, bias 2^47 per addend so every addend is positive and the sum never
+    // carries into the count).  Integer addition is associative, so the total does not depend
+    // on the order in which the workgroups arrive: the result is deterministic.  The workgroup
+    // whose add returns count == k_splits-1 is the last one for that output: it holds the
+    // complete sum, writes y and puts the word back to zero for the next launch.
+    if (active && (lane & 1) == 0 && out < a.n) {
+        const float scaled = fminf(fmaxf(total * 16777216.f, -1.4e14f), 1.4e14f);  // |v| < 2^47
+        const unsigned long long addend =
+            (unsigned long long)(__float2ll_rn(scaled) + (1ll << 47)) + (1ull << 56);
+        unsigned long long *word = a.accum + out;
+        const unsigned long long old =
+            __hip_atomic_fetch_add(word, addend, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if ((old >> 56) == (unsigned long long)(a.k_splits - 1)) {
+            const unsigned long long sum = (old + addend) & ((1ull << 56) - 1);
+            const long long value = (long long)sum - (long long)a.k_splits * (1ll << 47);
+            y[(size_t)out * a.y_stride] = __float2half_rn(__ll2float_rn(value) * (1.f / 16777216.f));
+            __hip_atomic_store(word, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         }
     }
-    if (tid == 0) a.counters[ntile] = 0u;  // ready for the next launch on this stream
 }
 
 // ------------------------------------------------------------------------------------------
