@@ -81,6 +81,8 @@ def main():
     ap.add_argument("--copies", type=int, default=17, help="distinct weight copies rotated through")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-dense", action="store_true", help="skip the dense fp16 GEMV comparator")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="also run a plain 256 MiB device copy (known traffic) for scaling rocprof byte counters")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build measures one GPU only (got --gpus %d); the path shards by output "
@@ -137,6 +139,14 @@ def main():
     mean_abs, max_abs, rel_l2 = oracle.error_stats(y, truth)
     ref_y = oracle.ref_kernel_fp16(w["bW"][:, :, :1024], w["alpha"].astype(np.float16)[:, :, :1024], None, x16[0])
     ref_err = oracle.error_stats(ref_y, truth[0, :1024])
+
+    if args.copy_calibration:
+        src = torch.empty(128 * 1024 * 1024, dtype=torch.float16, device=dev).fill_(1.0)  # 256 MiB
+        dst = torch.empty_like(src)
+        for _ in range(5):
+            torch.mul(src, 1.0, out=dst)  # an ordinary elementwise kernel: reads 256 MiB, writes 256 MiB
+        torch.cuda.synchronize()
+        del src, dst
 
     dense = None
     if not args.no_dense:

@@ -5,6 +5,7 @@
 #include <hip/hip_runtime_api.h>
 
 #include <cstdarg>
+#include <cstdint>
 #include <cstdio>
 #include <cstring>
 #include <new>
@@ -55,6 +56,8 @@ struct lutgemm_weight {
     uint16_t *d_scales;
     unsigned long long *d_accum;  // split-k accumulators, one 64-bit word per (padded) output
     size_t accum_bytes;
+    void *d_xrows;                // staging for column-batched activations, grown on demand
+    size_t xrows_bytes;
     Plan plan;
 };
 
@@ -190,21 +193,38 @@ int run_matvec(const lutgemm_weight *w, const void *x, void *y, int m, void *str
     a.blocks_per_split = w->plan.blocks_per_split;
     const uint16_t *xh = static_cast<const uint16_t *>(x);
     uint16_t *yh = static_cast<uint16_t *>(y);
+    if (((uintptr_t)x & 15u) != 0 || (!cols && m > 1 && (s.k % 8) != 0))
+        return fail(LUTGEMM_ERR_BAD_SHAPE, "x must be 16-byte aligned");
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    if (cols && m > 1) {
+        // gather the m columns into contiguous rows first (the kernel reads 16 bytes per lane)
+        lutgemm_weight *mw = const_cast<lutgemm_weight *>(w);
+        const size_t need = (size_t)m * s.k * sizeof(uint16_t);
+        if (mw->xrows_bytes < need) {
+            hipError_t e = hipStreamSynchronize(st);  // an earlier launch may still read the old buffer
+            if (e != hipSuccess) return hip_fail(e, "hipStreamSynchronize");
+            if (mw->d_xrows) (void)hipFree(mw->d_xrows);
+            mw->d_xrows = nullptr;
+            mw->xrows_bytes = 0;
+            e = hipMalloc(&mw->d_xrows, need);
+            if (e != hipSuccess) return hip_fail(e, "hipMalloc(column staging)");
+            mw->xrows_bytes = need;
+        }
+        hipError_t e = lutgemm_kernels::launch_gather_columns(x, mw->d_xrows, s.k, m, st);
+        if (e != hipSuccess) return hip_fail(e, "launch gather_columns_kernel");
+        xh = static_cast<const uint16_t *>(mw->d_xrows);
+    }
     for (int r = 0; r < m; r++) {
-        if (cols) {  // x [k][m], y [n][m]
-            a.x = xh + r;
+        a.x = xh + (size_t)r * s.k;
+        if (cols) {  // y [n][m]
             a.y = yh + r;
-            a.x_stride = m;
             a.y_stride = m;
-        } else {     // x [m][k], y [m][n]
-            a.x = xh + (size_t)r * s.k;
+        } else {     // y [m][n]
             a.y = yh + (size_t)r * s.n;
-            a.x_stride = 1;
             a.y_stride = 1;
         }
         hipError_t e = lutgemm_kernels::launch_matvec(s.q, s.has_offset, s.gsub, a,
-                                                      w->plan.ntiles * w->plan.k_splits, w->plan.waves,
-                                                      static_cast<hipStream_t>(stream));
+                                                      w->plan.ntiles * w->plan.k_splits, w->plan.waves, st);
         if (e != hipSuccess) return hip_fail(e, "launch lut_matvec_kernel");
     }
     return LUTGEMM_OK;
@@ -249,7 +269,7 @@ int lutgemm_weight_destroy(lutgemm_weight *w)
 {
     if (!w) return LUTGEMM_OK;
     int st = LUTGEMM_OK;
-    void *ptrs[3] = {w->d_signs, w->d_scales, w->d_accum};
+    void *ptrs[4] = {w->d_signs, w->d_scales, w->d_accum, w->d_xrows};
     for (void *p : ptrs)
         if (p) {
             hipError_t e = hipFree(p);

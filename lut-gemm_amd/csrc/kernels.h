@@ -11,7 +11,7 @@ namespace lutgemm_kernels {
 struct MatvecArgs {
     const uint8_t *signs;   // sign tiles (layout.h)
     const uint16_t *scales; // scale tiles (layout.h)
-    const void *x;          // fp16 activations, element i at x[i * x_stride]
+    const void *x;          // fp16 activations, contiguous, 16-byte aligned
     void *y;                // fp16 outputs, element j at y[j * y_stride]
     unsigned long long *accum;  // [nb*32] split-k accumulators (count | fixed-point sum), zero
                                 // between launches; used when k_splits > 1
@@ -20,7 +20,7 @@ struct MatvecArgs {
     int ntiles;             // column tiles = ceil(nb / waves)
     int k_splits;           // workgroups along k
     int blocks_per_split;   // k-blocks per workgroup
-    int x_stride, y_stride;
+    int y_stride;           // output j goes to y[j * y_stride]
 };
 
 struct DequantArgs {
@@ -34,6 +34,9 @@ struct DequantArgs {
 // workgroups = ntiles * k_splits, `waves` wavefronts of 64 lanes per workgroup.
 hipError_t launch_matvec(int q, int has_offset, int gsub, const MatvecArgs &a, int workgroups,
                          int waves, hipStream_t stream);
+
+// fp16 [k][m] -> [m][k]
+hipError_t launch_gather_columns(const void *cols, void *rows, int k, int m, hipStream_t stream);
 
 hipError_t launch_dequantize(const DequantArgs &a, hipStream_t stream);
 

@@ -523,6 +523,16 @@ __global__ __launch_bounds__(256) void dequantize_kernel(DequantArgs a)
     }
 }
 
+// x [k][m] (m vectors stored as columns) -> rows [m][k], so that the matvec kernel can read
+// each vector with 16-byte loads.
+__global__ __launch_bounds__(256) void gather_columns_kernel(const uint16_t *cols, uint16_t *rows, int k, int m)
+{
+    const size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx >= (size_t)k * m) return;
+    const int r = (int)(idx / k), i = (int)(idx % k);
+    rows[idx] = cols[(size_t)i * m + r];
+}
+
 template <int Q, bool OFF, int GSUB>
 hipError_t launch_one(const MatvecArgs &a, int workgroups, int threads, hipStream_t stream)
 {
@@ -579,6 +589,15 @@ hipError_t launch_matvec(int q, int has_offset, int gsub, const MatvecArgs &a, i
 #endif
         default: return hipErrorInvalidValue;
     }
+}
+
+hipError_t launch_gather_columns(const void *cols, void *rows, int k, int m, hipStream_t stream)
+{
+    const size_t total = (size_t)k * m;
+    const int threads = 256;
+    hipLaunchKernelGGL(gather_columns_kernel, dim3((unsigned)((total + threads - 1) / threads)), dim3(threads),
+                       0, stream, static_cast<const uint16_t *>(cols), static_cast<uint16_t *>(rows), k, m);
+    return hipGetLastError();
 }
 
 hipError_t launch_dequantize(const DequantArgs &a, hipStream_t stream)
