@@ -86,7 +86,7 @@ int lutgemm_weight_info(const lutgemm_weight *w, lutgemm_weight_info_t *info);
  * kernel::nqmv (mv_fp16.hpp:121) or kernel::nqmv_bias (mv_fp16_bias.hpp:143); here every
  * 1 <= m <= LUTGEMM_MAX_BATCH stays on the table-lookup kernel.
  * Calls that overlap in time on the same handle race on its split-K workspace. */
-#define LUTGEMM_MAX_BATCH 64
+#define LUTGEMM_MAX_BATCH 4096
 int lutgemm_matvec(const lutgemm_weight *w, const void *x, void *y, int m, void *stream);
 
 /* Column-batched form: x is [k][m] and y is [n][m] (m vectors stored as columns).

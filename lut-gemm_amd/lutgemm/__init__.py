@@ -21,7 +21,7 @@ LIB_PATH = os.path.join(os.path.dirname(_HERE), "liblutgemm_hip.so")
 
 OK = 0
 ERR_NULL_POINTER, ERR_BAD_SHAPE, ERR_NO_DEVICE, ERR_HIP, ERR_OUT_OF_MEMORY, ERR_UNSUPPORTED = range(1, 7)
-MAX_BATCH = 64
+MAX_BATCH = 4096
 
 # every symbol include/lutgemm_c.h declares
 EXPORTED = [
