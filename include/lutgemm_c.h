@@ -38,7 +38,7 @@ typedef enum lutgemm_status {
 } lutgemm_status;
 
 /* Opaque packed weight: device-resident sign tiles, scales and offsets plus the launch plan
- * and the split-K workspace.  Stands in for class lutGEMM::nQWeight_fp16
+ * and the split-k accumulators (one 64-bit word per output).  Stands in for class lutGEMM::nQWeight_fp16
  * (lutGEMM/include/nQWeight_fp16.h:27-52). */
 typedef struct lutgemm_weight lutgemm_weight;
 
@@ -79,20 +79,23 @@ int lutgemm_weight_info(const lutgemm_weight *w, lutgemm_weight_info_t *info);
 
 /* y[r][0..n) = x[r][0..k) * W for r < m, fp16 in / fp16 out, fp32 accumulation, asynchronous
  * on `stream` (a hipStream_t passed as void*, NULL = the default stream).  x and y are
- * device pointers, row-major [m][k] and [m][n].  The offset term is applied iff the weight
- * was created with q_bias.  No memset of y is needed and none is issued.
+ * device pointers, row-major [m][k] and [m][n], x 16-byte aligned.  The offset term is applied
+ * iff the weight was created with q_bias.  No memset of y is needed and none is issued; the
+ * call allocates nothing.  The result is deterministic (bit-identical from launch to launch).
  * Replaces lutGEMM::matmul(void* output, void* input, nQWeight_fp16&, int m, int algo)
  * (lutGEMM/include/kernels.h:27, lutGEMM/src/kernels.cu:64-71), which for m == 1 runs
  * kernel::nqmv (mv_fp16.hpp:121) or kernel::nqmv_bias (mv_fp16_bias.hpp:143); here every
  * 1 <= m <= LUTGEMM_MAX_BATCH stays on the table-lookup kernel.
- * Calls that overlap in time on the same handle race on its split-K workspace. */
+ * Calls that overlap in time on the same handle race on its split-k accumulators. */
 #define LUTGEMM_MAX_BATCH 4096
 int lutgemm_matvec(const lutgemm_weight *w, const void *x, void *y, int m, void *stream);
 
 /* Column-batched form: x is [k][m] and y is [n][m] (m vectors stored as columns).
  * Replaces lutGEMM::matmul(void* output, nQWeight_fp16&, void* input, int n, int algo)
  * (lutGEMM/include/kernels.h:26, lutGEMM/src/kernels.cu:56-63).  For m == 1 it is the same
- * operation as lutgemm_matvec. */
+ * operation as lutgemm_matvec.  For m > 1 the columns are first gathered into a staging buffer
+ * owned by the handle; the buffer is allocated (and the stream synchronised) the first time a
+ * given m is exceeded. */
 int lutgemm_matvec_cols(const lutgemm_weight *w, const void *x, void *y, int m, void *stream);
 
 /* `count` independent matvecs issued back to back on one stream with a single call (for a
@@ -119,8 +122,9 @@ int lutgemm_weight_unpack(const lutgemm_weight *w, uint32_t *bW, uint16_t *alpha
 int lutgemm_weight_plan(const lutgemm_weight *w, int *workgroups, int *waves_per_group,
                         int *k_splits, int *k_blocks_per_group);
 
-/* Override the launch plan (0 keeps the automatic choice for that field); reallocates the
- * split-K workspace.  Returns LUTGEMM_ERR_BAD_SHAPE if the request cannot be launched. */
+/* Override the launch plan (0 keeps the automatic choice for that field); synchronises the
+ * device first.  Returns LUTGEMM_ERR_BAD_SHAPE if the request cannot be launched
+ * (1..12 waves per workgroup, 1..min(k/512 rounded up, 128) k-splits). */
 int lutgemm_weight_set_plan(lutgemm_weight *w, int waves_per_group, int k_splits);
 
 /* Device pointers of the packed arrays, for the public data members of the C++ layer. */
