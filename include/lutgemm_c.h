@@ -127,6 +127,13 @@ int lutgemm_weight_plan(const lutgemm_weight *w, int *workgroups, int *waves_per
  * (1..12 waves per workgroup, 1..min(k/512 rounded up, 128) k-splits). */
 int lutgemm_weight_set_plan(lutgemm_weight *w, int waves_per_group, int k_splits);
 
+/* Measure the most promising launch plans on the device (a few launches each, on `stream`, with
+ * scratch activations of its own) and keep the fastest.  Optional: the automatic plan is chosen
+ * from a model, this replaces it by a measurement.  Synchronises `stream`; allocates and frees
+ * temporary device buffers.  No counterpart in the reference, whose tile sizes are fixed
+ * (lutGEMM/src/cuda/kernels/mv_fp16.hpp:122-124). */
+int lutgemm_weight_autotune(lutgemm_weight *w, void *stream);
+
 /* Device pointers of the packed arrays, for the public data members of the C++ layer. */
 int lutgemm_weight_device_ptrs(const lutgemm_weight *w, void **signs, void **scales, void **offsets);
 

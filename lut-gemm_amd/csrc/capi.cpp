@@ -4,6 +4,7 @@
 
 #include <hip/hip_runtime_api.h>
 
+#include <algorithm>
 #include <cstdarg>
 #include <cstdint>
 #include <cstdio>
@@ -63,37 +64,58 @@ struct lutgemm_weight {
 
 namespace {
 
-// Choose waves per workgroup and the k-split so that the workgroups fill the compute units
-// in as few, as full rounds as possible.  One workgroup owns `waves` batches of 32 outputs
-// and `blocks_per_split` k-blocks; it rebuilds one 64 KiB table set per k-block, so more
-// waves per workgroup amortise the build, and more k-blocks per workgroup amortise the final
-// cross-lane reduction and the split-k exchange.
+// Choose waves per workgroup and the k-split.  One workgroup owns `waves` batches of 32 outputs and
+// `blocks_per_split` k-blocks and occupies a compute unit by itself (128 KiB of LDS).  The model
+// below is in shader cycles and was fitted to measurements on MI355X: a workgroup pays a start-up
+// (first memory latency, first table build) and an end (cross-lane reduction, split-k atomic);
+// per k-block it needs the longer of the time to stream `waves` tiles at the compute unit's share
+// of HBM bandwidth and the LDS-bound time of the lookups.  Several rounds of workgroups pay the
+// start-up again, so one full round of fat workgroups usually wins over many small ones.
+double plan_cost(const Shape &s, int cus, int waves, int splits, Plan *out)
+{
+    const double kStart = 3000.0, kEnd = 1500.0;  // per workgroup
+    const double kFairBytes = 10.0;               // HBM bytes per cycle per CU when all CUs stream
+    const double kPeakBytes = 24.0;               // what one CU can pull when few CUs are active
+    const double kLookup = 2.3;                   // cycles per wave-level lookup (LDS bound)
+    const double kBuild = 450.0;                  // table build + barrier per k-block
+    const double kLatency = 6000.0;               // loaded HBM round trip
+    const double kGroup = 200.0;                  // one group of 8 lookups of a lone wavefront
+    const double tile_bytes = (double)sign_tile_bytes(s) + (double)scale_tile_bytes(s);
+    const double tile_lookups = 32.0 * s.q;
+    const int ntiles = div_up(s.nb, waves);
+    const int bps = div_up(s.ts, splits);
+    const int ks = div_up(s.ts, bps);
+    if (ks != splits) return -1.0;  // same plan as a smaller `splits`
+    const long wgs = (long)ntiles * ks;
+    const double rounds = (double)((wgs + cus - 1) / cus);
+    const double active = (double)(wgs < cus ? wgs : cus);
+    double bw = kFairBytes * cus / active;
+    if (bw > kPeakBytes) bw = kPeakBytes;
+    // a tile is requested one k-block ahead, so a k-block cannot take less than one memory
+    // round trip; one wavefront alone is bound by the LDS latency of its lookup groups
+    double t_mem = waves * tile_bytes / bw;
+    if (t_mem < kLatency) t_mem = kLatency;
+    double t_cmp = waves * tile_lookups * kLookup;
+    if (t_cmp < 4.0 * s.q * kGroup) t_cmp = 4.0 * s.q * kGroup;
+    t_cmp += kBuild;
+    const double t_wg = kStart + bps * (t_mem > t_cmp ? t_mem : t_cmp) + kEnd + (ks > 1 ? 1000.0 : 0.0);
+    *out = Plan{waves, ntiles, bps, ks};
+    return rounds * t_wg;
+}
+
 Plan choose_plan(const Shape &s, int cus)
 {
     Plan best{};
     double best_cost = 1e300;
-    // rough per-workgroup costs in SIMD issue slots (wave instructions per SIMD)
-    const double lookup = 2.0 * s.q * 16 * 3.2 + (s.has_offset ? 40 : 0);
-    for (int waves = 1; waves <= kMaxWaves; waves++) {
-        const int ntiles = div_up(s.nb, waves);
-        const double per_simd = (double)div_up(waves, 4);
+    for (int waves = 1; waves <= kMaxWaves; waves++)
         for (int splits = 1; splits <= s.ts && splits <= kMaxSplits; splits++) {
-            const int bps = div_up(s.ts, splits);
-            const int ks = div_up(s.ts, bps);
-            if (ks != splits) continue;  // same plan as a smaller `splits`
-            const long wgs = (long)ntiles * ks;
-            const double rounds = (double)((wgs + cus - 1) / cus);
-            const double build = 160.0 + 40.0;  // quarter build + barriers
-            double wg_cost = bps * (build + per_simd * lookup) + per_simd * 180.0;
-            if (ks > 1) wg_cost += 150.0;  // split-k atomic round trip
-            // padding waste: wavefronts beyond the last batch still stream a tile
-            const double cost = rounds * wg_cost;
-            if (cost < best_cost - 1e-9) {
+            Plan p;
+            const double cost = plan_cost(s, cus, waves, splits, &p);
+            if (cost >= 0.0 && cost < best_cost - 1e-9) {
                 best_cost = cost;
-                best = Plan{waves, ntiles, bps, ks};
+                best = p;
             }
         }
-    }
     return best;
 }
 
@@ -391,6 +413,60 @@ int lutgemm_weight_set_plan(lutgemm_weight *w, int waves_per_group, int k_splits
     if (e != hipSuccess) return hip_fail(e, "hipDeviceSynchronize");
     w->plan = p;
     return alloc_workspace(w);
+}
+
+int lutgemm_weight_autotune(lutgemm_weight *w, void *stream)
+{
+    if (!w) return fail(LUTGEMM_ERR_NULL_POINTER, "null argument to weight_autotune");
+    const Shape &s = w->shape;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    // candidates: the best plans of the model, measured on the device
+    struct Cand { double cost; Plan p; };
+    std::vector<Cand> cands;
+    for (int waves = 1; waves <= kMaxWaves; waves++)
+        for (int splits = 1; splits <= s.ts && splits <= kMaxSplits; splits++) {
+            Plan p;
+            const double cost = plan_cost(s, w->compute_units, waves, splits, &p);
+            if (cost >= 0.0) cands.push_back(Cand{cost, p});
+        }
+    std::sort(cands.begin(), cands.end(), [](const Cand &a, const Cand &b) { return a.cost < b.cost; });
+    if (cands.size() > 24) cands.resize(24);
+
+    void *x = nullptr, *y = nullptr;
+    hipEvent_t e0 = nullptr, e1 = nullptr;
+    int status = LUTGEMM_OK;
+    hipError_t e = hipMalloc(&x, (size_t)s.k * 2);
+    if (e == hipSuccess) e = hipMalloc(&y, (size_t)s.n * 2);
+    if (e == hipSuccess) e = hipMemsetAsync(x, 0, (size_t)s.k * 2, st);
+    if (e == hipSuccess) e = hipEventCreate(&e0);
+    if (e == hipSuccess) e = hipEventCreate(&e1);
+    if (e != hipSuccess) status = hip_fail(e, "autotune setup");
+    const Plan before = w->plan;
+    Plan best = before;
+    float best_ms = 1e30f;
+    const int reps = 8;
+    for (size_t i = 0; status == LUTGEMM_OK && i < cands.size(); i++) {
+        w->plan = cands[i].p;
+        for (int r = 0; r < 2 && status == LUTGEMM_OK; r++) status = run_matvec(w, x, y, 1, stream, false);
+        if (status != LUTGEMM_OK) break;
+        e = hipEventRecord(e0, st);
+        for (int r = 0; r < reps && status == LUTGEMM_OK; r++) status = run_matvec(w, x, y, 1, stream, false);
+        if (e == hipSuccess) e = hipEventRecord(e1, st);
+        if (e == hipSuccess) e = hipEventSynchronize(e1);
+        float ms = 0.f;
+        if (e == hipSuccess) e = hipEventElapsedTime(&ms, e0, e1);
+        if (e != hipSuccess) status = hip_fail(e, "autotune timing");
+        if (status == LUTGEMM_OK && ms < best_ms) {
+            best_ms = ms;
+            best = cands[i].p;
+        }
+    }
+    w->plan = status == LUTGEMM_OK ? best : before;
+    if (e0) (void)hipEventDestroy(e0);
+    if (e1) (void)hipEventDestroy(e1);
+    if (x) (void)hipFree(x);
+    if (y) (void)hipFree(y);
+    return status;
 }
 
 int lutgemm_weight_device_ptrs(const lutgemm_weight *w, void **signs, void **scales, void **offsets)

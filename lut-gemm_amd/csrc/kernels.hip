@@ -429,10 +429,10 @@ __global__ __launch_bounds__(768) void lut_matvec_kernel(MatvecArgs a)
         const int cur = (ts - ts0) & 1;
         const float chunk_sum = ((f[0] + f[1]) + (f[2] + f[3])) + ((f[4] + f[5]) + (f[6] + f[7]));
         const bool more = ts + 1 < ts1;
-        // table set of the next k-block (all zero activations past the end: harmless, unused)
+        // table set of the next k-block, if there is one
         unpack_activations(xnext, f);
         xnext = load_activations(x, a.k, ts + 2, lane, ts + 2 < ts1);
-        build_tables(table + (cur ^ 1) * kTableFloats, f, lane, wave, waves);
+        if (more) build_tables(table + (cur ^ 1) * kTableFloats, f, lane, wave, waves);
         process_tile<Q, OFF, GSUB>(tile, lane_base + (uint32_t)cur * (kTableFloats * 4u), chunk_sum, acc,
                                    tile_address<Q, QO, GSUB>(signs, scales, tile0 + ts + 1, lane, more));
         // the next table set is complete and every lookup into the current one has finished

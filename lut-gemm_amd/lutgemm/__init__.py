@@ -27,7 +27,7 @@ MAX_BATCH = 4096
 EXPORTED = [
     "lutgemm_weight_create", "lutgemm_weight_create_f16", "lutgemm_weight_destroy", "lutgemm_weight_info",
     "lutgemm_matvec", "lutgemm_matvec_cols", "lutgemm_matvec_many", "lutgemm_dequantize", "lutgemm_weight_unpack",
-    "lutgemm_weight_plan", "lutgemm_weight_set_plan", "lutgemm_weight_device_ptrs", "lutgemm_packed_sizes",
+    "lutgemm_weight_plan", "lutgemm_weight_set_plan", "lutgemm_weight_autotune", "lutgemm_weight_device_ptrs", "lutgemm_packed_sizes",
     "lutgemm_pack_host", "lutgemm_unpack_host", "lutgemm_float_to_half", "lutgemm_last_error",
     "lutgemm_status_string", "lutgemm_version",
 ]
@@ -82,6 +82,7 @@ def load():
     L.lutgemm_weight_unpack.argtypes = [vp, vp, vp, vp]
     L.lutgemm_weight_plan.argtypes = [vp, pi, pi, pi, pi]
     L.lutgemm_weight_set_plan.argtypes = [vp, i, i]
+    L.lutgemm_weight_autotune.argtypes = [vp, vp]
     L.lutgemm_weight_device_ptrs.argtypes = [vp, pp, pp, pp]
     L.lutgemm_packed_sizes.argtypes = [i, i, i, i, i, psz, psz]
     L.lutgemm_pack_host.argtypes = [vp, vp, vp, i, i, i, i, vp, vp]
@@ -190,6 +191,11 @@ class BCQWeight:
 
     def set_plan(self, waves=0, k_splits=0):
         _check(load().lutgemm_weight_set_plan(self._h, waves, k_splits))
+
+    def autotune(self, stream=0):
+        """Measure candidate launch plans on the device and keep the fastest; returns the plan."""
+        _check(load().lutgemm_weight_autotune(self._h, stream or None))
+        return self.plan()
 
     def weight_bytes(self):
         """Algorithmic packed-weight bytes: signs + scales + offsets (unpadded)."""

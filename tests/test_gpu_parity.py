@@ -153,6 +153,21 @@ def test_every_launch_plan_agrees(lutgemm, oracle, device):
     W.close()
 
 
+def test_autotune_keeps_results_and_picks_a_valid_plan(lutgemm, oracle, device):
+    import torch
+    from lutgemm import synth
+    k, n, q, g = 4096, 2048, 3, 128
+    w, W = make(lutgemm, synth, k, n, q, g, offset=True, seed=21)
+    x = synth.make_x(1, k, seed=21)
+    truth = truth_of(oracle, w, x)
+    say("case autotune")
+    plan = W.autotune(torch.cuda.current_stream().cuda_stream)
+    assert 1 <= plan["waves"] <= 12 and 1 <= plan["k_splits"] <= 8
+    assert plan["workgroups"] == -(-(n // 32) // plan["waves"]) * plan["k_splits"]
+    assert_within_tolerance(run_matvec(lutgemm, W, x, device), truth, "after autotune %s" % plan)
+    W.close()
+
+
 def test_back_to_back_launches_reuse_workspace(lutgemm, oracle, device):
     """The split-k arrival counters reset themselves: many launches on one stream stay correct."""
     import torch
