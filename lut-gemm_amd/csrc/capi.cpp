@@ -122,7 +122,7 @@ Plan choose_plan(const Shape &s, int cus)
 int alloc_workspace(lutgemm_weight *w)
 {
     if (w->d_accum) return LUTGEMM_OK;  // size depends on the shape only
-    w->accum_bytes = (size_t)w->shape.nb * kBatch * sizeof(unsigned long long);
+    w->accum_bytes = 2 * (size_t)w->shape.nb * kBatch * sizeof(unsigned long long);  // two rows per pass
     hipError_t e = hipMalloc((void **)&w->d_accum, w->accum_bytes);
     if (e != hipSuccess) return hip_fail(e, "hipMalloc(split-k accumulators)");
     e = hipMemset(w->d_accum, 0, w->accum_bytes);
@@ -236,14 +236,20 @@ int run_matvec(const lutgemm_weight *w, const void *x, void *y, int m, void *str
         if (e != hipSuccess) return hip_fail(e, "launch gather_columns_kernel");
         xh = static_cast<const uint16_t *>(mw->d_xrows);
     }
-    for (int r = 0; r < m; r++) {
+    // two activation rows per pass over the weight, a last single row if m is odd
+    a.x_row_stride = s.k;
+    a.accum_row_stride = (long long)s.nb * kBatch;
+    for (int r = 0; r < m; r += 2) {
+        a.rows = m - r >= 2 ? 2 : 1;
         a.x = xh + (size_t)r * s.k;
         if (cols) {  // y [n][m]
             a.y = yh + r;
             a.y_stride = m;
+            a.y_row_stride = 1;
         } else {     // y [m][n]
             a.y = yh + (size_t)r * s.n;
             a.y_stride = 1;
+            a.y_row_stride = s.n;
         }
         hipError_t e = lutgemm_kernels::launch_matvec(s.q, s.has_offset, s.gsub, a,
                                                       w->plan.ntiles * w->plan.k_splits, w->plan.waves, st);

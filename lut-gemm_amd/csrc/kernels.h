@@ -13,7 +13,7 @@ struct MatvecArgs {
     const uint16_t *scales; // scale tiles (layout.h)
     const void *x;          // fp16 activations, contiguous, 16-byte aligned
     void *y;                // fp16 outputs, element j at y[j * y_stride]
-    unsigned long long *accum;  // [nb*32] split-k accumulators (count | fixed-point sum), zero
+    unsigned long long *accum;  // [2][nb*32] split-k accumulators (count | fixed-point sum), zero
                                 // between launches; used when k_splits > 1
     int k, n;
     int ts, nb;             // k-blocks, output batches
@@ -21,6 +21,10 @@ struct MatvecArgs {
     int k_splits;           // workgroups along k
     int blocks_per_split;   // k-blocks per workgroup
     int y_stride;           // output j goes to y[j * y_stride]
+    // rows == 2: a second activation row at x + x_row_stride goes to y + y_row_stride in the
+    // same pass (strides in fp16 elements), with its accumulators at accum + accum_row_stride
+    int rows;
+    long long x_row_stride, y_row_stride, accum_row_stride;
 };
 
 struct DequantArgs {

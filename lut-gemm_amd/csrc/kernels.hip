@@ -202,6 +202,116 @@ __device__ __forceinline__ void build_part(float *col, int part, const float (&f
     }
 }
 
+// ------------------------------------------------------------------------------------------
+// Two activation rows per pass.  The table set holds, for every (entry, lane), the partial sums
+// of both rows side by side (8 bytes), laid out [lane / 32][entry][lane % 32]: the address is
+// still three bytes of lane constant around the sign byte (one v_perm_b32), a lookup is one
+// ds_read_b64, and the 16 lanes served per LDS cycle read 16 consecutive 8-byte slots, so the
+// reads stay conflict free.  Each weight byte fetched from HBM now serves two rows; per row and
+// lookup the cost drops to 1.5 vector ALU instructions and half an LDS read.  Table values,
+// their order of accumulation and the reduction are those of the one-row kernel, so each row's
+// result is bit-identical to a one-row launch with the same plan.
+//
+// The 64-bit read results are named in C++ (a register pair cannot be split inside an asm
+// template), so the reads and their multiply-adds are separate asm statements and the first
+// one waits for all of its reads.
+// ------------------------------------------------------------------------------------------
+constexpr int kTable2Floats = 2 * kTableFloats;  // 128 KiB
+
+#define LG2_FMA(k, v, CTRL) "v_fmac_f32_dpp %" #k ", %16, %" #v CTRL
+#define LG2_OPS(acc0, acc1, I0, t)                                                                       \
+    "+v"(acc0[I0 + 0]), "+v"(acc0[I0 + 1]), "+v"(acc0[I0 + 2]), "+v"(acc0[I0 + 3]), "+v"(acc1[I0 + 0]),   \
+        "+v"(acc1[I0 + 1]), "+v"(acc1[I0 + 2]), "+v"(acc1[I0 + 3])                                        \
+        : "v"((uint32_t)t[0]), "v"((uint32_t)(t[0] >> 32)), "v"((uint32_t)t[1]),                           \
+          "v"((uint32_t)(t[1] >> 32)), "v"((uint32_t)t[2]), "v"((uint32_t)(t[2] >> 32)),                   \
+          "v"((uint32_t)t[3]), "v"((uint32_t)(t[3] >> 32))
+
+// acc0/acc1[I0..I0+3] += scale * (row 0 / row 1 half of t[0..3]); I0 a multiple of 4, scale
+// register s holds the scales of these four outputs (see lookup8 for where in the row).
+// Operands: %0-%3 row 0 accumulators, %4-%7 row 1, %8-%15 values, %16 scale, %17.. lane numbers.
+template <int GSUB, int I0>
+__device__ __forceinline__ void fma4x2(float (&acc0)[kBatch], float (&acc1)[kBatch],
+                                       const unsigned long long (&t)[4], float s)
+{
+    if constexpr (GSUB == 1) {
+        constexpr int L = I0 % 16;
+#define LG2_CTRL(n) " row_newbcast:%" #n " row_mask:0xf bank_mask:0xf\n"
+        asm volatile("s_nop 1\n" LG2_FMA(0, 8, LG2_CTRL(17)) LG2_FMA(4, 9, LG2_CTRL(17))
+                     LG2_FMA(1, 10, LG2_CTRL(18)) LG2_FMA(5, 11, LG2_CTRL(18))
+                     LG2_FMA(2, 12, LG2_CTRL(19)) LG2_FMA(6, 13, LG2_CTRL(19))
+                     LG2_FMA(3, 14, LG2_CTRL(20)) LG2_FMA(7, 15, LG2_CTRL(20))
+                     : LG2_OPS(acc0, acc1, I0, t), "v"(s), "n"(L), "n"(L + 1), "n"(L + 2), "n"(L + 3));
+#undef LG2_CTRL
+    } else if constexpr (GSUB == 2) {
+        constexpr int L = I0 % 8;
+#define LG2_LO(n) " row_newbcast:%" #n " row_mask:0xf bank_mask:0x3\n"
+#define LG2_HI(n) " row_newbcast:%" #n " row_mask:0xf bank_mask:0xc\n"
+        asm volatile("s_nop 1\n"
+                     LG2_FMA(0, 8, LG2_LO(17)) LG2_FMA(0, 8, LG2_HI(21)) LG2_FMA(4, 9, LG2_LO(17)) LG2_FMA(4, 9, LG2_HI(21))
+                     LG2_FMA(1, 10, LG2_LO(18)) LG2_FMA(1, 10, LG2_HI(22)) LG2_FMA(5, 11, LG2_LO(18)) LG2_FMA(5, 11, LG2_HI(22))
+                     LG2_FMA(2, 12, LG2_LO(19)) LG2_FMA(2, 12, LG2_HI(23)) LG2_FMA(6, 13, LG2_LO(19)) LG2_FMA(6, 13, LG2_HI(23))
+                     LG2_FMA(3, 14, LG2_LO(20)) LG2_FMA(3, 14, LG2_HI(24)) LG2_FMA(7, 15, LG2_LO(20)) LG2_FMA(7, 15, LG2_HI(24))
+                     : LG2_OPS(acc0, acc1, I0, t), "v"(s), "n"(L), "n"(L + 1), "n"(L + 2), "n"(L + 3),
+                       "n"(L + 8), "n"(L + 9), "n"(L + 10), "n"(L + 11));
+#undef LG2_LO
+#undef LG2_HI
+    } else {
+        asm volatile("s_nop 1\n" LG2_FMA(0, 8, LG_QUAD(0)) LG2_FMA(4, 9, LG_QUAD(0))
+                     LG2_FMA(1, 10, LG_QUAD(1)) LG2_FMA(5, 11, LG_QUAD(1))
+                     LG2_FMA(2, 12, LG_QUAD(2)) LG2_FMA(6, 13, LG_QUAD(2))
+                     LG2_FMA(3, 14, LG_QUAD(3)) LG2_FMA(7, 15, LG_QUAD(3))
+                     : LG2_OPS(acc0, acc1, I0, t), "v"(s));
+    }
+}
+
+// Eight two-row lookups: outputs I0..I0+7 (I0 a multiple of 8), sign bytes in w0 and w1.
+template <int GSUB, int I0>
+__device__ __forceinline__ void lookup8x2(float (&acc0)[kBatch], float (&acc1)[kBatch], uint32_t w0,
+                                          uint32_t w1, uint32_t lane_off, float sa, float sb)
+{
+    unsigned long long ta[4], tb[4];
+    uint32_t ad[8];
+    asm volatile(
+        "v_perm_b32 %8, %16, %18, %19\n v_perm_b32 %9, %16, %18, %20\n v_perm_b32 %10, %16, %18, %21\n"
+        "v_perm_b32 %11, %16, %18, %22\n v_perm_b32 %12, %17, %18, %19\n v_perm_b32 %13, %17, %18, %20\n"
+        "v_perm_b32 %14, %17, %18, %21\n v_perm_b32 %15, %17, %18, %22\n"
+        "ds_read_b64 %0, %8\n ds_read_b64 %1, %9\n ds_read_b64 %2, %10\n ds_read_b64 %3, %11\n"
+        "ds_read_b64 %4, %12\n ds_read_b64 %5, %13\n ds_read_b64 %6, %14\n ds_read_b64 %7, %15\n"
+        "s_waitcnt lgkmcnt(0)\n"
+        : "=&v"(ta[0]), "=&v"(ta[1]), "=&v"(ta[2]), "=&v"(ta[3]), "=&v"(tb[0]), "=&v"(tb[1]), "=&v"(tb[2]),
+          "=&v"(tb[3]), "=&v"(ad[0]), "=&v"(ad[1]), "=&v"(ad[2]), "=&v"(ad[3]), "=&v"(ad[4]), "=&v"(ad[5]),
+          "=&v"(ad[6]), "=&v"(ad[7])
+        : LG_IN(w0, w1, lane_off)
+        : "memory");
+    fma4x2<GSUB, I0>(acc0, acc1, ta, sa);
+    fma4x2<GSUB, I0 + 4>(acc0, acc1, tb, GSUB == 4 ? sb : sa);
+}
+
+// build_part for two rows: entries are (row 0, row 1) pairs, 32 pairs per entry row.
+__device__ __forceinline__ void build_part2(float2 *col, int part, const float (&f0)[8], const float (&f1)[8])
+{
+    float lo0[8], lo1[8];
+#pragma unroll
+    for (int t = 0; t < 8; t++) {
+        lo0[t] = ((t & 1) ? f0[0] : -f0[0]) + ((t & 2) ? f0[1] : -f0[1]) + ((t & 4) ? f0[2] : -f0[2]);
+        lo1[t] = ((t & 1) ? f1[0] : -f1[0]) + ((t & 2) ? f1[1] : -f1[1]) + ((t & 4) ? f1[2] : -f1[2]);
+    }
+    const float top0 =
+        (((part & 1) ? f0[5] : -f0[5]) + ((part & 2) ? f0[6] : -f0[6])) + ((part & 4) ? f0[7] : -f0[7]);
+    const float top1 =
+        (((part & 1) ? f1[5] : -f1[5]) + ((part & 2) ? f1[6] : -f1[6])) + ((part & 4) ? f1[7] : -f1[7]);
+    float2 *q = col + part * (32 * 32);
+#pragma unroll
+    for (int h = 0; h < 4; h++) {
+        const float hi0 = top0 + (((h & 1) ? f0[3] : -f0[3]) + ((h & 2) ? f0[4] : -f0[4]));
+        const float hi1 = top1 + (((h & 1) ? f1[3] : -f1[3]) + ((h & 2) ? f1[4] : -f1[4]));
+#pragma unroll
+        for (int t = 0; t < 8; t++) q[(h * 8 + t) * 32] = make_float2(hi0 + lo0[t], hi1 + lo1[t]);
+        __builtin_amdgcn_sched_barrier(0);
+    }
+}
+
+
 template <int Q, int QO, int GSUB>
 struct TileRegs {
     u32x4 sign[2 * Q];
@@ -380,6 +490,37 @@ __device__ __forceinline__ float reduce_across_lanes(float (&acc)[kBatch], int l
     return acc[0] + as_f(other);
 }
 
+// Lane pair (2j, 2j+1) of a wavefront holds the k-range total of output `out`; the even lane
+// delivers it.  With one k-split it is the result.  Otherwise: one 64-bit atomic add per output,
+// no barrier, no second pass.  The word holds an arrival count in its top 8 bits and the running
+// sum below it, as a biased fixed-point integer (2^-24 units, bias 2^47 per addend so every
+// addend is positive and the sum never carries into the count).  Integer addition is
+// associative, so the total does not depend on the order in which the workgroups arrive: the
+// result is deterministic.  The workgroup whose add returns count == k_splits-1 is the last one
+// for that output: it holds the complete sum, writes y and puts the word back to zero for the
+// next launch.
+__device__ __forceinline__ void finish_output(float total, bool active, int out, int lane, __half *y,
+                                              unsigned long long *accum, const MatvecArgs &a)
+{
+    if (!(active && (lane & 1) == 0 && out < a.n)) return;
+    if (a.k_splits == 1) {
+        y[(size_t)out * a.y_stride] = __float2half_rn(total);
+        return;
+    }
+    const float scaled = fminf(fmaxf(total * 16777216.f, -1.4e14f), 1.4e14f);  // |v| < 2^47
+    const unsigned long long addend =
+        (unsigned long long)(__float2ll_rn(scaled) + (1ll << 47)) + (1ull << 56);
+    unsigned long long *word = accum + out;
+    const unsigned long long old =
+        __hip_atomic_fetch_add(word, addend, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    if ((old >> 56) == (unsigned long long)(a.k_splits - 1)) {
+        const unsigned long long sum = (old + addend) & ((1ull << 56) - 1);
+        const long long value = (long long)sum - (long long)a.k_splits * (1ll << 47);
+        y[(size_t)out * a.y_stride] = __float2half_rn(__ll2float_rn(value) * (1.f / 16777216.f));
+        __hip_atomic_store(word, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+}
+
 template <int Q, bool OFF, int GSUB>
 __global__ __launch_bounds__(768) void lut_matvec_kernel(MatvecArgs a)
 {
@@ -440,35 +581,114 @@ __global__ __launch_bounds__(768) void lut_matvec_kernel(MatvecArgs a)
     }
 
     const float total = reduce_across_lanes(acc, lane);
+    finish_output(total, active, nb * kBatch + (lane >> 1), lane, reinterpret_cast<__half *>(a.y), a.accum, a);
+}
+
+// process_tile for two activation rows (tables of lookup8x2).
+template <int Q, bool OFF, int GSUB>
+__device__ __forceinline__ void process_tile2(TileRegs<Q, Q + (OFF ? 1 : 0), GSUB> &t, uint32_t lane_off,
+                                              float chunk_sum0, float chunk_sum1, float (&acc0)[kBatch],
+                                              float (&acc1)[kBatch], const NextTile &next)
+{
+    constexpr int QO = Q + (OFF ? 1 : 0);
+    constexpr int NSC = 2 * GSUB * QO;
+    constexpr int SUBL = 16 / GSUB;
+    float sc[NSC];
+#pragma unroll
+    for (int d = 0; d < GSUB * QO; d++) {
+        const __half2 h2 = *reinterpret_cast<const __half2 *>(&t.scale[d]);
+        sc[2 * d] = __low2float(h2);
+        sc[2 * d + 1] = __high2float(h2);
+    }
+#pragma unroll
+    for (int d = 0; d < GSUB * QO; d++) t.scale[d] = __builtin_nontemporal_load(next.scale + d);
+    auto sa = [&](auto I0, int bo) { return sc[(I0 / SUBL) * QO + bo]; };
+    auto sb = [&](auto I0, int bo) { return sc[((I0 + 4) / SUBL) * QO + bo]; };
+
+    if constexpr (OFF) {
+        static_for<4>([&](auto G) {
+            constexpr int I0 = G * 8;
+            offset8<GSUB, I0>(acc0, chunk_sum0, sa(std::integral_constant<int, I0>{}, Q),
+                              sb(std::integral_constant<int, I0>{}, Q));
+            offset8<GSUB, I0>(acc1, chunk_sum1, sa(std::integral_constant<int, I0>{}, Q),
+                              sb(std::integral_constant<int, I0>{}, Q));
+        });
+    }
+
+    static_for<2 * Q>([&](auto U) {
+        constexpr int b = U / 2, h = U % 2;
+        constexpr int I0 = h * 16;
+        const u32x4 w4 = t.sign[U];
+        lookup8x2<GSUB, I0>(acc0, acc1, w4.x, w4.y, lane_off, sa(std::integral_constant<int, I0>{}, b),
+                            sb(std::integral_constant<int, I0>{}, b));
+        lookup8x2<GSUB, I0 + 8>(acc0, acc1, w4.z, w4.w, lane_off, sa(std::integral_constant<int, I0 + 8>{}, b),
+                                sb(std::integral_constant<int, I0 + 8>{}, b));
+        t.sign[U] = __builtin_nontemporal_load(next.sign + U * next.sign_stride);
+    });
+}
+
+// Two activation rows (a.x and a.x + a.x_row_stride) against the same weight in one pass over
+// its tiles.  One 128 KiB table set: it is rebuilt between two barriers at the start of every
+// k-block, while the tile loads of that block (issued one block earlier) are in flight.
+template <int Q, bool OFF, int GSUB>
+__global__ __launch_bounds__(768) void lut_matvec2_kernel(MatvecArgs a)
+{
+    constexpr int QO = Q + (OFF ? 1 : 0);
+    __shared__ float2 table[kTable2Floats / 2];
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int waves = blockDim.x >> 6;
+    const int ntile = blockIdx.x % a.ntiles;
+    const int ks = blockIdx.x / a.ntiles;
+    const int nb = ntile * waves + wave;
+    const bool active = nb < a.nb;
+    const int ts0 = ks * a.blocks_per_split;
+    const int ts1 = min(ts0 + a.blocks_per_split, a.ts);
+
+    const u32x4 *signs = reinterpret_cast<const u32x4 *>(a.signs);
+    const uint32_t *scales = reinterpret_cast<const uint32_t *>(a.scales);
+    const __half *x0 = reinterpret_cast<const __half *>(a.x);
+    const __half *x1 = x0 + a.x_row_stride;
+
+    float acc0[kBatch], acc1[kBatch];
+#pragma unroll
+    for (int i = 0; i < kBatch; i++) acc0[i] = acc1[i] = 0.f;
+
+    // bytes 0, 2 and 3 of every lookup address: (lane % 32) * 8 + (lane / 32) * 64 KiB + LDS base
+    const uint32_t lane_base = (uint32_t)(lane & 31) * 8u + ((uint32_t)(lane >> 5) << 16) +
+                               (uint32_t)(size_t)(__attribute__((address_space(3))) float2 *)table;
+    float2 *col = table + (lane >> 5) * (256 * 32) + (lane & 31);
+    const size_t tile0 = (size_t)(active ? nb : 0) * a.ts;
+
+    TileRegs<Q, QO, GSUB> tile;
+    u32x4 xa = load_activations(x0, a.k, ts0, lane, true);
+    u32x4 xb = load_activations(x1, a.k, ts0, lane, true);
+    load_tile(tile, tile_address<Q, QO, GSUB>(signs, scales, tile0 + ts0, lane, true));
+
+    for (int ts = ts0; ts < ts1; ts++) {
+        float f0[8], f1[8];
+        unpack_activations(xa, f0);
+        unpack_activations(xb, f1);
+        const float chunk_sum0 = ((f0[0] + f0[1]) + (f0[2] + f0[3])) + ((f0[4] + f0[5]) + (f0[6] + f0[7]));
+        const float chunk_sum1 = ((f1[0] + f1[1]) + (f1[2] + f1[3])) + ((f1[4] + f1[5]) + (f1[6] + f1[7]));
+        const bool more = ts + 1 < ts1;
+        xa = load_activations(x0, a.k, ts + 1, lane, more);
+        xb = load_activations(x1, a.k, ts + 1, lane, more);
+        __syncthreads();  // every lookup into the previous table set has finished
+        for (int task = wave; task < kBuildParts; task += waves) build_part2(col, task, f0, f1);
+        __syncthreads();
+        process_tile2<Q, OFF, GSUB>(tile, lane_base, chunk_sum0, chunk_sum1, acc0, acc1,
+                                    tile_address<Q, QO, GSUB>(signs, scales, tile0 + ts + 1, lane, more));
+    }
 
     const int out = nb * kBatch + (lane >> 1);
     __half *y = reinterpret_cast<__half *>(a.y);
-    if (a.k_splits == 1) {
-        if (active && (lane & 1) == 0 && out < a.n) y[(size_t)out * a.y_stride] = __float2half_rn(total);
-        return;
-    }
-
-    // split-k: one 64-bit atomic add per output, no barrier, no second pass.  The word holds an
-    // arrival count in its top 8 bits and the running sum below it, as a biased fixed-point
-    // integer (2^-24 units, bias 2^47 per addend so every addend is positive and the sum never
-    // carries into the count).  Integer addition is associative, so the total does not depend
-    // on the order in which the workgroups arrive: the result is deterministic.  The workgroup
-    // whose add returns count == k_splits-1 is the last one for that output: it holds the
-    // complete sum, writes y and puts the word back to zero for the next launch.
-    if (active && (lane & 1) == 0 && out < a.n) {
-        const float scaled = fminf(fmaxf(total * 16777216.f, -1.4e14f), 1.4e14f);  // |v| < 2^47
-        const unsigned long long addend =
-            (unsigned long long)(__float2ll_rn(scaled) + (1ll << 47)) + (1ull << 56);
-        unsigned long long *word = a.accum + out;
-        const unsigned long long old =
-            __hip_atomic_fetch_add(word, addend, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        if ((old >> 56) == (unsigned long long)(a.k_splits - 1)) {
-            const unsigned long long sum = (old + addend) & ((1ull << 56) - 1);
-            const long long value = (long long)sum - (long long)a.k_splits * (1ll << 47);
-            y[(size_t)out * a.y_stride] = __float2half_rn(__ll2float_rn(value) * (1.f / 16777216.f));
-            __hip_atomic_store(word, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        }
-    }
+    const float total0 = reduce_across_lanes(acc0, lane);
+    finish_output(total0, active, out, lane, y, a.accum, a);
+    const float total1 = reduce_across_lanes(acc1, lane);
+    finish_output(total1, active && a.rows > 1, out, lane, y + a.y_row_stride, a.accum + a.accum_row_stride, a);
 }
 
 // ------------------------------------------------------------------------------------------
@@ -536,7 +756,10 @@ __global__ __launch_bounds__(256) void gather_columns_kernel(const uint16_t *col
 template <int Q, bool OFF, int GSUB>
 hipError_t launch_one(const MatvecArgs &a, int workgroups, int threads, hipStream_t stream)
 {
-    hipLaunchKernelGGL((lut_matvec_kernel<Q, OFF, GSUB>), dim3(workgroups), dim3(threads), 0, stream, a);
+    if (a.rows > 1)
+        hipLaunchKernelGGL((lut_matvec2_kernel<Q, OFF, GSUB>), dim3(workgroups), dim3(threads), 0, stream, a);
+    else
+        hipLaunchKernelGGL((lut_matvec_kernel<Q, OFF, GSUB>), dim3(workgroups), dim3(threads), 0, stream, a);
     return hipGetLastError();
 }
 
