@@ -34,7 +34,8 @@ typedef enum lutgemm_status {
     LUTGEMM_ERR_NO_DEVICE = 3,     /* no HIP device / the device is not usable */
     LUTGEMM_ERR_HIP = 4,           /* a HIP runtime call failed; see lutgemm_last_error() */
     LUTGEMM_ERR_OUT_OF_MEMORY = 5, /* host or device allocation failed */
-    LUTGEMM_ERR_UNSUPPORTED = 6    /* valid request outside what this build implements */
+    LUTGEMM_ERR_UNSUPPORTED = 6,   /* valid request outside what this build implements */
+    LUTGEMM_ERR_IO = 7             /* a packed-weight file could not be read or written */
 } lutgemm_status;
 
 /* Opaque packed weight: device-resident sign tiles, scales and offsets plus the launch plan
@@ -154,6 +155,34 @@ int lutgemm_pack_host(const uint32_t *bW, const uint16_t *alpha, const uint16_t 
 /* Exact inverse of lutgemm_pack_host; any of bW / alpha / q_bias may be NULL. */
 int lutgemm_unpack_host(const void *signs, const void *scales, int k, int n, int q, int num_groups,
                         int has_offset, uint32_t *bW, uint16_t *alpha, uint16_t *q_bias);
+
+/* ---- packed-weight files ------------------------------------------------------------------
+ * The reference has no on-disk form of a packed weight: its Python examples only print the
+ * converted tensors (examples/quant_model_rtn.py:86-99) and nQWeight_fp16::parsing re-reads host
+ * arrays on every start (lutGEMM/src/nQWeight_fp16.cu:60-91).  A file written here holds the
+ * device tiling itself (64-byte header: magic "LUTGEMMW", format version, tile layout id, k, n,
+ * q, num_groups, has_offset, byte counts; then the sign tiles, then the scale tiles, all little
+ * endian), so loading is one read and two copies to the device, with no packing work. */
+
+/* Host only: pack host arrays (as for lutgemm_weight_create_f16) straight into a file. */
+int lutgemm_pack_file(const uint32_t *bW, const uint16_t *alpha, const uint16_t *q_bias, int k, int n, int q,
+                      int num_groups, const char *path);
+
+/* Host only: read a file back into the host input layout; any of bW / alpha / q_bias may be
+ * NULL, `info` (optional) receives the shape, so a first call with NULL arrays sizes a second. */
+int lutgemm_unpack_file(const char *path, uint32_t *bW, uint16_t *alpha, uint16_t *q_bias,
+                        lutgemm_weight_info_t *info);
+
+/* Write the packed weight held by a handle / create a handle on the current device from a
+ * file.  LUTGEMM_ERR_IO if the file cannot be opened, is not such a file, was written for
+ * another tile layout or is truncated.  Synchronous. */
+int lutgemm_weight_save(const lutgemm_weight *w, const char *path);
+int lutgemm_weight_load(const char *path, lutgemm_weight **out);
+
+/* A second, independent handle with its own device copy of the packed weight and its own
+ * workspace (device-to-device copy, no packing), with the same launch plan.  Handles must not
+ * be shared by launches that overlap in time; clones can be. */
+int lutgemm_weight_clone(const lutgemm_weight *w, lutgemm_weight **out);
 
 /* float -> binary16 bit patterns, round to nearest even: the conversion applied to alpha and
  * q_bias at ingest (stands for the __float2half loops of lutGEMM/src/nQWeight_fp16.cu:81,85). */

@@ -130,15 +130,11 @@ int alloc_workspace(lutgemm_weight *w)
     return LUTGEMM_OK;
 }
 
-int create_common(const uint32_t *bW, const uint16_t *alpha_h, const uint16_t *q_bias_h, int k, int n,
-                  int q, int num_groups, lutgemm_weight **out)
+// New handle for shape s on the current device from tiles already in the device layout
+// (host or device memory, `kind` says which).
+int create_from_tiles(const Shape &s, const void *signs, const void *scales, hipMemcpyKind kind,
+                      lutgemm_weight **out)
 {
-    Shape s;
-    if (!make_shape(k, n, q, num_groups, q_bias_h != nullptr, &s))
-        return fail(LUTGEMM_ERR_BAD_SHAPE,
-                    "bad shape k=%d n=%d q=%d num_groups=%d (need k%%32==0, 1<=q<=8, "
-                    "k%%num_groups==0, (k/num_groups)%%32==0)",
-                    k, n, q, num_groups);
     int count = 0;
     hipError_t e = hipGetDeviceCount(&count);
     if (e != hipSuccess || count <= 0)
@@ -158,17 +154,6 @@ int create_common(const uint32_t *bW, const uint16_t *alpha_h, const uint16_t *q
     w->compute_units = prop.multiProcessorCount > 0 ? prop.multiProcessorCount : 256;
 
     const size_t sb = sign_bytes(s), cb = scale_bytes(s);
-    std::vector<uint8_t> signs;
-    std::vector<uint16_t> scales;
-    try {
-        signs.resize(sb);
-        scales.resize(cb / 2);
-    } catch (const std::bad_alloc &) {
-        delete w;
-        return fail(LUTGEMM_ERR_OUT_OF_MEMORY, "host staging allocation failed (%zu bytes)", sb + cb);
-    }
-    lutgemm_packer::pack(s, bW, alpha_h, q_bias_h, signs.data(), scales.data());
-
     int st = LUTGEMM_OK;
     e = hipMalloc((void **)&w->d_signs, sb);
     if (e != hipSuccess) st = hip_fail(e, "hipMalloc(signs)");
@@ -177,11 +162,11 @@ int create_common(const uint32_t *bW, const uint16_t *alpha_h, const uint16_t *q
         if (e != hipSuccess) st = hip_fail(e, "hipMalloc(scales)");
     }
     if (st == LUTGEMM_OK) {
-        e = hipMemcpy(w->d_signs, signs.data(), sb, hipMemcpyHostToDevice);
+        e = hipMemcpy(w->d_signs, signs, sb, kind);
         if (e != hipSuccess) st = hip_fail(e, "hipMemcpy(signs)");
     }
     if (st == LUTGEMM_OK) {
-        e = hipMemcpy(w->d_scales, scales.data(), cb, hipMemcpyHostToDevice);
+        e = hipMemcpy(w->d_scales, scales, cb, kind);
         if (e != hipSuccess) st = hip_fail(e, "hipMemcpy(scales)");
     }
     if (st == LUTGEMM_OK) {
@@ -194,6 +179,124 @@ int create_common(const uint32_t *bW, const uint16_t *alpha_h, const uint16_t *q
     }
     *out = w;
     return LUTGEMM_OK;
+}
+
+void fill_info(const Shape &s, size_t accum_bytes, lutgemm_weight_info_t *info)
+{
+    info->k = s.k;
+    info->n = s.n;
+    info->q = s.q;
+    info->num_groups = s.num_groups;
+    info->group_size = s.group_size;
+    info->has_offset = s.has_offset;
+    info->sign_bytes = (size_t)s.k / 8 * s.q * s.n;
+    info->scale_bytes = (size_t)s.num_groups * s.q * s.n * 2;
+    info->offset_bytes = s.has_offset ? (size_t)s.num_groups * s.n * 2 : 0;
+    info->device_bytes = sign_bytes(s) + scale_bytes(s) + accum_bytes;
+}
+
+int shape_or_fail(int k, int n, int q, int num_groups, bool has_offset, Shape *s)
+{
+    if (!make_shape(k, n, q, num_groups, has_offset, s))
+        return fail(LUTGEMM_ERR_BAD_SHAPE,
+                    "bad shape k=%d n=%d q=%d num_groups=%d (need k%%32==0, 1<=q<=8, "
+                    "k%%num_groups==0, (k/num_groups)%%32==0)",
+                    k, n, q, num_groups);
+    return LUTGEMM_OK;
+}
+
+int pack_to_host(const Shape &s, const uint32_t *bW, const uint16_t *alpha_h, const uint16_t *q_bias_h,
+                 std::vector<uint8_t> *signs, std::vector<uint16_t> *scales)
+{
+    try {
+        signs->resize(sign_bytes(s));
+        scales->resize(scale_bytes(s) / 2);
+    } catch (const std::bad_alloc &) {
+        return fail(LUTGEMM_ERR_OUT_OF_MEMORY, "host staging allocation failed (%zu bytes)",
+                    sign_bytes(s) + scale_bytes(s));
+    }
+    lutgemm_packer::pack(s, bW, alpha_h, q_bias_h, signs->data(), scales->data());
+    return LUTGEMM_OK;
+}
+
+int create_common(const uint32_t *bW, const uint16_t *alpha_h, const uint16_t *q_bias_h, int k, int n,
+                  int q, int num_groups, lutgemm_weight **out)
+{
+    Shape s;
+    int st = shape_or_fail(k, n, q, num_groups, q_bias_h != nullptr, &s);
+    if (st != LUTGEMM_OK) return st;
+    std::vector<uint8_t> signs;
+    std::vector<uint16_t> scales;
+    st = pack_to_host(s, bW, alpha_h, q_bias_h, &signs, &scales);
+    if (st != LUTGEMM_OK) return st;
+    return create_from_tiles(s, signs.data(), scales.data(), hipMemcpyHostToDevice, out);
+}
+
+// Packed-weight file: 64-byte little-endian header, the sign tiles, the scale tiles.
+constexpr char kFileMagic[8] = {'L', 'U', 'T', 'G', 'E', 'M', 'M', 'W'};
+constexpr uint32_t kFileVersion = 1;
+// identifies the tile layout: lanes, chunk, batch (a file written for another tiling is refused)
+constexpr uint32_t kFileLayout = (uint32_t)kLanes | ((uint32_t)kChunk << 8) | ((uint32_t)kBatch << 16);
+struct FileHeader {
+    char magic[8];
+    uint32_t version, layout;
+    uint32_t k, n, q, num_groups, has_offset, reserved;
+    uint64_t sign_bytes, scale_bytes;
+    uint64_t pad[1];
+};
+static_assert(sizeof(FileHeader) == 64, "file header is 64 bytes");
+
+int write_file(const char *path, const Shape &s, const void *signs, const void *scales)
+{
+    FILE *f = std::fopen(path, "wb");
+    if (!f) return fail(LUTGEMM_ERR_IO, "cannot open %s for writing", path);
+    FileHeader h{};
+    std::memcpy(h.magic, kFileMagic, 8);
+    h.version = kFileVersion;
+    h.layout = kFileLayout;
+    h.k = (uint32_t)s.k;
+    h.n = (uint32_t)s.n;
+    h.q = (uint32_t)s.q;
+    h.num_groups = (uint32_t)s.num_groups;
+    h.has_offset = (uint32_t)s.has_offset;
+    h.sign_bytes = sign_bytes(s);
+    h.scale_bytes = scale_bytes(s);
+    bool ok = std::fwrite(&h, sizeof(h), 1, f) == 1;
+    ok = ok && std::fwrite(signs, 1, h.sign_bytes, f) == h.sign_bytes;
+    ok = ok && std::fwrite(scales, 1, h.scale_bytes, f) == h.scale_bytes;
+    ok = (std::fclose(f) == 0) && ok;
+    if (!ok) return fail(LUTGEMM_ERR_IO, "short write to %s", path);
+    return LUTGEMM_OK;
+}
+
+int read_file(const char *path, Shape *s, std::vector<uint8_t> *signs, std::vector<uint16_t> *scales)
+{
+    FILE *f = std::fopen(path, "rb");
+    if (!f) return fail(LUTGEMM_ERR_IO, "cannot open %s", path);
+    FileHeader h{};
+    int st = LUTGEMM_OK;
+    if (std::fread(&h, sizeof(h), 1, f) != 1 || std::memcmp(h.magic, kFileMagic, 8) != 0)
+        st = fail(LUTGEMM_ERR_IO, "%s is not a packed-weight file", path);
+    else if (h.version != kFileVersion || h.layout != kFileLayout)
+        st = fail(LUTGEMM_ERR_IO, "%s: file version %u / layout 0x%x, this library reads %u / 0x%x", path,
+                  h.version, h.layout, kFileVersion, kFileLayout);
+    else if (h.k > 0x7fffffffu || h.n > 0x7fffffffu ||
+             !make_shape((int)h.k, (int)h.n, (int)h.q, (int)h.num_groups, h.has_offset != 0, s) ||
+             h.sign_bytes != sign_bytes(*s) || h.scale_bytes != scale_bytes(*s))
+        st = fail(LUTGEMM_ERR_IO, "%s: inconsistent header", path);
+    if (st == LUTGEMM_OK) {
+        try {
+            signs->resize(h.sign_bytes);
+            scales->resize(h.scale_bytes / 2);
+        } catch (const std::bad_alloc &) {
+            st = fail(LUTGEMM_ERR_OUT_OF_MEMORY, "host staging allocation failed");
+        }
+    }
+    if (st == LUTGEMM_OK && (std::fread(signs->data(), 1, h.sign_bytes, f) != h.sign_bytes ||
+                             std::fread(scales->data(), 1, h.scale_bytes, f) != h.scale_bytes))
+        st = fail(LUTGEMM_ERR_IO, "%s is truncated", path);
+    std::fclose(f);
+    return st;
 }
 
 int run_matvec(const lutgemm_weight *w, const void *x, void *y, int m, void *stream, bool cols)
@@ -293,6 +396,73 @@ int lutgemm_weight_create(const uint32_t *bW, const float *alpha, const float *q
     return create_common(bW, ah.data(), q_bias ? zh.data() : nullptr, k, n, q, num_groups, out);
 }
 
+int lutgemm_weight_clone(const lutgemm_weight *w, lutgemm_weight **out)
+{
+    if (!w || !out) return fail(LUTGEMM_ERR_NULL_POINTER, "null argument to weight_clone");
+    int st = create_from_tiles(w->shape, w->d_signs, w->d_scales, hipMemcpyDeviceToDevice, out);
+    if (st == LUTGEMM_OK) (*out)->plan = w->plan;
+    return st;
+}
+
+int lutgemm_weight_save(const lutgemm_weight *w, const char *path)
+{
+    if (!w || !path) return fail(LUTGEMM_ERR_NULL_POINTER, "null argument to weight_save");
+    const Shape &s = w->shape;
+    std::vector<uint8_t> signs;
+    std::vector<uint16_t> scales;
+    try {
+        signs.resize(sign_bytes(s));
+        scales.resize(scale_bytes(s) / 2);
+    } catch (const std::bad_alloc &) {
+        return fail(LUTGEMM_ERR_OUT_OF_MEMORY, "host staging allocation failed");
+    }
+    hipError_t e = hipMemcpy(signs.data(), w->d_signs, signs.size(), hipMemcpyDeviceToHost);
+    if (e != hipSuccess) return hip_fail(e, "hipMemcpy(signs)");
+    e = hipMemcpy(scales.data(), w->d_scales, scales.size() * 2, hipMemcpyDeviceToHost);
+    if (e != hipSuccess) return hip_fail(e, "hipMemcpy(scales)");
+    return write_file(path, s, signs.data(), scales.data());
+}
+
+int lutgemm_weight_load(const char *path, lutgemm_weight **out)
+{
+    if (!path || !out) return fail(LUTGEMM_ERR_NULL_POINTER, "null argument to weight_load");
+    Shape s;
+    std::vector<uint8_t> signs;
+    std::vector<uint16_t> scales;
+    int st = read_file(path, &s, &signs, &scales);
+    if (st != LUTGEMM_OK) return st;
+    return create_from_tiles(s, signs.data(), scales.data(), hipMemcpyHostToDevice, out);
+}
+
+int lutgemm_pack_file(const uint32_t *bW, const uint16_t *alpha, const uint16_t *q_bias, int k, int n, int q,
+                      int num_groups, const char *path)
+{
+    if (!bW || !alpha || !path) return fail(LUTGEMM_ERR_NULL_POINTER, "null argument to pack_file");
+    Shape s;
+    int st = shape_or_fail(k, n, q, num_groups, q_bias != nullptr, &s);
+    if (st != LUTGEMM_OK) return st;
+    std::vector<uint8_t> signs;
+    std::vector<uint16_t> scales;
+    st = pack_to_host(s, bW, alpha, q_bias, &signs, &scales);
+    if (st != LUTGEMM_OK) return st;
+    return write_file(path, s, signs.data(), scales.data());
+}
+
+int lutgemm_unpack_file(const char *path, uint32_t *bW, uint16_t *alpha, uint16_t *q_bias,
+                        lutgemm_weight_info_t *info)
+{
+    if (!path) return fail(LUTGEMM_ERR_NULL_POINTER, "null argument to unpack_file");
+    Shape s;
+    std::vector<uint8_t> signs;
+    std::vector<uint16_t> scales;
+    int st = read_file(path, &s, &signs, &scales);
+    if (st != LUTGEMM_OK) return st;
+    if (info) fill_info(s, 0, info);
+    if (bW || alpha || q_bias)
+        lutgemm_packer::unpack(s, signs.data(), scales.data(), bW, alpha, s.has_offset ? q_bias : nullptr);
+    return LUTGEMM_OK;
+}
+
 int lutgemm_weight_destroy(lutgemm_weight *w)
 {
     if (!w) return LUTGEMM_OK;
@@ -310,17 +480,7 @@ int lutgemm_weight_destroy(lutgemm_weight *w)
 int lutgemm_weight_info(const lutgemm_weight *w, lutgemm_weight_info_t *info)
 {
     if (!w || !info) return fail(LUTGEMM_ERR_NULL_POINTER, "null argument to weight_info");
-    const Shape &s = w->shape;
-    info->k = s.k;
-    info->n = s.n;
-    info->q = s.q;
-    info->num_groups = s.num_groups;
-    info->group_size = s.group_size;
-    info->has_offset = s.has_offset;
-    info->sign_bytes = (size_t)s.k / 8 * s.q * s.n;
-    info->scale_bytes = (size_t)s.num_groups * s.q * s.n * 2;
-    info->offset_bytes = s.has_offset ? (size_t)s.num_groups * s.n * 2 : 0;
-    info->device_bytes = sign_bytes(s) + scale_bytes(s) + w->accum_bytes;
+    fill_info(w->shape, w->accum_bytes, info);
     return LUTGEMM_OK;
 }
 
@@ -542,6 +702,7 @@ const char *lutgemm_status_string(int status)
         case LUTGEMM_ERR_HIP: return "HIP runtime error";
         case LUTGEMM_ERR_OUT_OF_MEMORY: return "out of memory";
         case LUTGEMM_ERR_UNSUPPORTED: return "unsupported";
+        case LUTGEMM_ERR_IO: return "file input/output failed";
         default: return "unknown status";
     }
 }

@@ -576,8 +576,9 @@ __global__ __launch_bounds__(768) void lut_matvec_kernel(MatvecArgs a)
         if (more) build_tables(table + (cur ^ 1) * kTableFloats, f, lane, wave, waves);
         process_tile<Q, OFF, GSUB>(tile, lane_base + (uint32_t)cur * (kTableFloats * 4u), chunk_sum, acc,
                                    tile_address<Q, QO, GSUB>(signs, scales, tile0 + ts + 1, lane, more));
-        // the next table set is complete and every lookup into the current one has finished
-        __syncthreads();
+        // the next table set is complete and every lookup into the current one has finished;
+        // after the last k-block each wavefront goes straight to its reduction
+        if (more) __syncthreads();
     }
 
     const float total = reduce_across_lanes(acc, lane);

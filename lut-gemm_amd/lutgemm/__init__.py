@@ -20,7 +20,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(os.path.dirname(_HERE), "liblutgemm_hip.so")
 
 OK = 0
-ERR_NULL_POINTER, ERR_BAD_SHAPE, ERR_NO_DEVICE, ERR_HIP, ERR_OUT_OF_MEMORY, ERR_UNSUPPORTED = range(1, 7)
+ERR_NULL_POINTER, ERR_BAD_SHAPE, ERR_NO_DEVICE, ERR_HIP, ERR_OUT_OF_MEMORY, ERR_UNSUPPORTED, ERR_IO = range(1, 8)
 MAX_BATCH = 4096
 
 # every symbol include/lutgemm_c.h declares
@@ -29,7 +29,8 @@ EXPORTED = [
     "lutgemm_matvec", "lutgemm_matvec_cols", "lutgemm_matvec_many", "lutgemm_dequantize", "lutgemm_weight_unpack",
     "lutgemm_weight_plan", "lutgemm_weight_set_plan", "lutgemm_weight_autotune", "lutgemm_weight_device_ptrs", "lutgemm_packed_sizes",
     "lutgemm_pack_host", "lutgemm_unpack_host", "lutgemm_float_to_half", "lutgemm_last_error",
-    "lutgemm_status_string", "lutgemm_version",
+    "lutgemm_status_string", "lutgemm_version", "lutgemm_pack_file", "lutgemm_unpack_file", "lutgemm_weight_save",
+    "lutgemm_weight_load", "lutgemm_weight_clone",
 ]
 
 
@@ -81,6 +82,11 @@ def load():
     L.lutgemm_dequantize.argtypes = [vp, vp, i, vp]
     L.lutgemm_weight_unpack.argtypes = [vp, vp, vp, vp]
     L.lutgemm_weight_plan.argtypes = [vp, pi, pi, pi, pi]
+    L.lutgemm_pack_file.argtypes = [vp, vp, vp, i, i, i, i, ctypes.c_char_p]
+    L.lutgemm_unpack_file.argtypes = [ctypes.c_char_p, vp, vp, vp, ctypes.POINTER(WeightInfo)]
+    L.lutgemm_weight_save.argtypes = [vp, ctypes.c_char_p]
+    L.lutgemm_weight_load.argtypes = [ctypes.c_char_p, pp]
+    L.lutgemm_weight_clone.argtypes = [vp, pp]
     L.lutgemm_weight_set_plan.argtypes = [vp, i, i]
     L.lutgemm_weight_autotune.argtypes = [vp, vp]
     L.lutgemm_weight_device_ptrs.argtypes = [vp, pp, pp, pp]
@@ -146,6 +152,30 @@ def unpack_host(signs, scales, k, n, q, num_groups, has_offset):
     return bW, alpha, q_bias
 
 
+def pack_file(path, bW, alpha, k, n, q, num_groups=1, q_bias=None):
+    """Host only: write a packed-weight file from arrays in the reference layout."""
+    bW = np.ascontiguousarray(bW, np.uint32)
+    a = float_to_half_bits(alpha) if np.asarray(alpha).dtype != np.float16 else np.ascontiguousarray(alpha).view(np.uint16)
+    z = None
+    if q_bias is not None:
+        z = float_to_half_bits(q_bias) if np.asarray(q_bias).dtype != np.float16 else np.ascontiguousarray(q_bias).view(np.uint16)
+    if bW.size != (k // 32) * q * n or a.size != num_groups * q * n or (z is not None and z.size != num_groups * n):
+        raise LutGemmError(ERR_BAD_SHAPE, "array sizes do not match k=%d n=%d q=%d num_groups=%d" % (k, n, q, num_groups))
+    _check(load().lutgemm_pack_file(_ptr(bW), _ptr(a), _ptr(z), k, n, q, num_groups, os.fsencode(path)))
+
+
+def unpack_file(path):
+    """Host only: packed-weight file -> dict(bW uint32, alpha float16, q_bias float16|None, k, n, q, num_groups)."""
+    info = WeightInfo()
+    _check(load().lutgemm_unpack_file(os.fsencode(path), None, None, None, ctypes.byref(info)))
+    bW = np.empty((info.k // 32, info.q, info.n), np.uint32)
+    alpha = np.empty((info.num_groups, info.q, info.n), np.uint16)
+    q_bias = np.empty((info.num_groups, info.n), np.uint16) if info.has_offset else None
+    _check(load().lutgemm_unpack_file(os.fsencode(path), _ptr(bW), _ptr(alpha), _ptr(q_bias), None))
+    return dict(bW=bW, alpha=alpha.view(np.float16), q_bias=q_bias.view(np.float16) if q_bias is not None else None,
+                k=info.k, n=info.n, q=info.q, num_groups=info.num_groups)
+
+
 class BCQWeight:
     """Packed BCQ weight on the current HIP device (the nQWeight_fp16 of this library).
 
@@ -174,10 +204,36 @@ class BCQWeight:
             z = np.ascontiguousarray(q_bias, np.float32) if q_bias is not None else None
             st = L.lutgemm_weight_create(_ptr(bW), _ptr(a), _ptr(z), k, n, q, num_groups, ctypes.byref(self._h))
         _check(st)
+        self._read_info()
+
+    def _read_info(self):
         info = self.info()
         self.kSize, self.mSize, self.nb = info.k, info.n, info.q
         self.num_groups, self.group_size = info.num_groups, info.group_size
         self.has_offset = bool(info.has_offset)
+
+    @classmethod
+    def _from_handle(cls, handle):
+        self = cls.__new__(cls)
+        self._h = handle
+        self._read_info()
+        return self
+
+    @classmethod
+    def load(cls, path):
+        """Handle on the current device from a packed-weight file (no packing work)."""
+        h = ctypes.c_void_p()
+        _check(load().lutgemm_weight_load(os.fsencode(path), ctypes.byref(h)))
+        return cls._from_handle(h)
+
+    def save(self, path):
+        _check(load().lutgemm_weight_save(self._h, os.fsencode(path)))
+
+    def clone(self):
+        """Independent handle with its own device copy and workspace, same launch plan."""
+        h = ctypes.c_void_p()
+        _check(load().lutgemm_weight_clone(self._h, ctypes.byref(h)))
+        return BCQWeight._from_handle(h)
 
     def info(self):
         info = WeightInfo()
