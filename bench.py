@@ -1,10 +1,10 @@
 #!/usr/bin/env python3
 """Benchmark of the BCQ LUT matvec on one MI355X.
 
-  python bench.py [--gpus 1] [--steps K] [--warmup W]
+  python bench.py [--gpus 1] [--steps K] [--warmup W] [--config cfg1]
 
-A step is one matvec of the headline configuration (cfg1: m=1, k=n=12288, q=3, g=128, fp16
-activations, no offset) with the packed weight already resident in HBM.  Consecutive steps use
+Default (cfg1, the headline): a step is one matvec of m=1, k=n=12288, q=3, g=128, fp16
+activations, no offset, with the packed weight already resident in HBM.  Consecutive steps use
 different weight copies (R copies, R * packed bytes > 4 x the 256 MiB last-level cache), so every
 step streams its weight from HBM and not from cache.  The K timed steps are issued back to back
 with one C-ABI call and bracketed by HIP events on the launch stream.
@@ -12,10 +12,18 @@ with one C-ABI call and bracketed by HIP events on the launch stream.
 Prints ONE JSON line: value = packed-weight GB/s (higher is better), plus us per matvec, the
 roofline block for the matvec kernel, the dense fp16 GEMV comparator, the single-copy ("hot")
 figure and the CPU baseline (the reference's CPU path restated in oracle/, timed on this box's
-host cores on a bounded slice of the same workload).
+host cores: the whole cfg0 matvec and a bounded slice of cfg1).
+
+Other workloads, same protocol, one JSON line each (no CPU / dense legs):
+  --config cfg0 | cfg2        single shapes
+  --config cfg3               k=n=7168, q in 1..4 x g in {32,64,128,k}: 16 points
+  --config cfg4 [--m M] [--graph]
+                              q=2 g=128 decoder layer: QKV, out, FC1, FC2 matvecs back to back,
+                              m activation rows; --graph replays the chain from a captured HIP graph
 """
 import argparse
 import json
+import math
 import os
 import sys
 import time
@@ -26,7 +34,12 @@ for _p in (ROOT, os.path.join(ROOT, "lut-gemm_amd")):
         sys.path.insert(0, _p)
 
 HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published peak
+LLC_BYTES = 256 << 20  # last-level (memory-side) cache
 METRIC = "µs/matvec + weight-GB/s (% HBM peak), n=k=12288 q=3 g=128 m=1 fp16"
+# HBM bytes per cfg1 launch from the rocprofv3 counter runs summarised in
+# profiles/lut_matvec_kernel_cfg1.md (FETCH_SIZE and WRITE_SIZE, scaled by the factors a plain
+# copy kernel of known size reads on the same counters)
+CFG1_MEASURED_TRAFFIC_BYTES = 64.9e6
 
 
 def event_time_ms(torch, fn, stream):
@@ -39,26 +52,40 @@ def event_time_ms(torch, fn, stream):
     return start.elapsed_time(stop)
 
 
-def cpu_baseline(cfg, x16, w, slice_n=12288):
-    """The reference's CPU path (dequantize_cpu then the float triple-loop matmul), restated in
-    oracle/, single-threaded as the reference is, on the first `slice_n` outputs of the workload;
-    then the same loops with OpenMP over all host cores."""
+def cpu_matvec(oracle, w, x16, slice_n, omp):
+    """dequantize_cpu then the fp32 triple-loop matmul (the reference's CPU path) on the first
+    slice_n outputs; returns (seconds, y, threads)."""
     import numpy as np
-    from oracle import oracle
-    k, n = cfg["k"], cfg["n"]
     bW = np.ascontiguousarray(w["bW"][:, :, :slice_n])
     alpha = np.ascontiguousarray(w["alpha"].astype(np.float16)[:, :, :slice_n])
     t0 = time.perf_counter()
-    fW = oracle.dequantize_cpu(bW, alpha)
-    y = oracle.matmul_cpu(x16, fW)
-    t1 = time.perf_counter()
-    fW2, threads = oracle.dequantize_cpu_omp(bW, alpha)
-    y2, _ = oracle.matmul_cpu_omp(x16, fW2)
-    t2 = time.perf_counter()
+    if omp:
+        fW, threads = oracle.dequantize_cpu_omp(bW, alpha)
+        y, _ = oracle.matmul_cpu_omp(x16, fW)
+    else:
+        fW, threads = oracle.dequantize_cpu(bW, alpha), 1
+        y = oracle.matmul_cpu(x16, fW)
+    return time.perf_counter() - t0, y, int(threads)
+
+
+def cpu_baseline(synth, cfg, x16, w, truth, slice_n=12288):
+    """The reference's CPU path restated in oracle/, single-threaded as the reference is, on the
+    first `slice_n` outputs of the cfg1 workload; then the same loops with OpenMP over the host
+    cores; then the whole cfg0 matvec (the reference's CPU-runnable configuration) both ways."""
+    import numpy as np
+    from oracle import oracle
+    k, n = cfg["k"], cfg["n"]
+    serial_s, y, _ = cpu_matvec(oracle, w, x16, slice_n, omp=False)
+    omp_s, _, threads = cpu_matvec(oracle, w, x16, slice_n, omp=True)
     scale = n / float(slice_n)
     b_w = (k * slice_n * cfg["q"] // 8) + (k // cfg["g"]) * cfg["q"] * slice_n * 2
-    serial_s = t1 - t0
-    omp_s = t2 - t1
+    c0 = synth.CONFIGS["cfg0"]
+    w0 = synth.make_weight(c0["k"], c0["n"], c0["q"], c0["g"], seed=0)
+    x0 = synth.make_x(1, c0["k"], seed=0)
+    b_w0, _ = synth.algorithmic_bytes(c0["k"], c0["n"], c0["q"], c0["g"], False, 1)
+    s0, y0, _ = cpu_matvec(oracle, w0, x0, c0["n"], omp=False)
+    o0, _, _ = cpu_matvec(oracle, w0, x0, c0["n"], omp=True)
+    t0 = oracle.matvec_f64(w0["bW"], w0["alpha"].astype(np.float16), None, x0)
     return {
         "value": b_w / serial_s / 1e9,
         "unit": "GB/s (packed-weight bytes)",
@@ -67,82 +94,127 @@ def cpu_baseline(cfg, x16, w, slice_n=12288):
         "sample": "cfg1 outputs 0..%d of %d (%.1f%% of one matvec): dequantize_cpu + matmul_cpu, %.2f s" % (
             slice_n - 1, n, 100.0 / scale, serial_s),
         "us_per_matvec_extrapolated": serial_s * scale * 1e6,
-        "openmp": {"cores": int(threads), "value": b_w / omp_s / 1e9,
+        "openmp": {"cores": threads, "value": b_w / omp_s / 1e9,
                    "us_per_matvec_extrapolated": omp_s * scale * 1e6},
+        "max_abs_vs_truth": float(np.abs(y[0].astype(np.float64) - truth[0, :y.shape[1]]).max()),
+        "cfg0_whole_matvec": {"us_per_matvec": s0 * 1e6, "value": b_w0 / s0 / 1e9,
+                              "openmp_us_per_matvec": o0 * 1e6, "openmp_value": b_w0 / o0 / 1e9,
+                              "max_abs_vs_truth": float(np.abs(y0.astype(np.float64) - t0).max())},
         "checksum": float(np.abs(y).sum()),
-    }, y
+    }
 
 
-def main():
-    ap = argparse.ArgumentParser()
-    ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=400)
-    ap.add_argument("--warmup", type=int, default=40)
-    ap.add_argument("--copies", type=int, default=17, help="distinct weight copies rotated through")
-    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
-    ap.add_argument("--no-dense", action="store_true", help="skip the dense fp16 GEMV comparator")
-    ap.add_argument("--copy-calibration", action="store_true",
-                    help="also run a plain 256 MiB device copy (known traffic) for scaling rocprof byte counters")
-    args = ap.parse_args()
-    if args.gpus != 1:
-        sys.exit("bench.py: this build measures one GPU only (got --gpus %d); the path shards by output "
-                 "columns, see DESIGN.md" % args.gpus)
+class Point:
+    """One weight shape on the device: R rotating copies, an autotuned plan, buffers."""
 
-    import numpy as np
-    import torch
+    def __init__(self, lutgemm, synth, torch, dev, k, n, q, g, rtn, m, seed, stream_handle, copies=None,
+                 rotation_bytes=4 * LLC_BYTES):
+        self.k, self.n, self.q, self.g, self.m = k, n, q, g, m
+        self.w = synth.make_weight(k, n, q, g, rtn=rtn, seed=seed)
+        self.has_offset = self.w["q_bias"] is not None
+        self.b_w, self.b_total = synth.algorithmic_bytes(k, n, q, g, self.has_offset, m)
+        if copies is None:
+            copies = min(200, max(2, int(math.ceil(rotation_bytes / float(self.b_w))) + 1))
+        self.copies = copies
+        first = lutgemm.BCQWeight(self.w["bW"], self.w["alpha"], k, n, q, k // g, self.w["q_bias"])
+        first.autotune(stream_handle)  # measured once (a few untimed launches); clones keep the plan
+        self.weights = [first] + [first.clone() for _ in range(copies - 1)]
+        self.x16 = synth.make_x(m, k, seed=seed)
+        self.xd = torch.from_numpy(self.x16).to(dev)
+        self.yd = torch.zeros((copies, m, n), dtype=torch.float16, device=dev)
+        self.plan = first.plan()
 
-    import lutgemm
-    from lutgemm import synth
+    def items(self, count, rotate=True, offset=0):
+        out = []
+        for i in range(count):
+            c = ((i + offset) % self.copies) if rotate else 0
+            out.append((self.weights[c], self.xd.data_ptr(), self.yd[c].data_ptr(), self.m))
+        return out
 
-    lutgemm.load()  # no fallback: fails loudly if the HIP library is not built
-    dev = torch.device("cuda:0")
-    torch.cuda.set_device(dev)
-    stream = torch.cuda.current_stream()
+    def parity(self, max_outputs=None):
+        """Error statistics of copy 0's last output against the fp64 oracle (checker only)."""
+        import numpy as np
+        from oracle import oracle
+        n_chk = self.n if max_outputs is None else min(self.n, max_outputs)
+        z = self.w["q_bias"].astype(np.float16)[:, :n_chk] if self.has_offset else None
+        truth = oracle.matvec_f64(np.ascontiguousarray(self.w["bW"][:, :, :n_chk]),
+                                  np.ascontiguousarray(self.w["alpha"].astype(np.float16)[:, :, :n_chk]),
+                                  np.ascontiguousarray(z) if z is not None else None, self.x16)
+        y = self.yd[0].cpu().numpy()[:, :n_chk]
+        mean_abs, max_abs, rel_l2 = oracle.error_stats(y, truth)
+        return {"truth": "fp64 accumulation over fp16-rounded inputs (oracle)", "outputs_checked": n_chk,
+                "mean_abs": mean_abs, "max_abs": max_abs, "rel_l2": rel_l2}, truth
+
+    def close(self):
+        for wgt in self.weights:
+            wgt.close()
+
+
+def time_point(lutgemm, torch, stream, pt, steps, warmup):
     sh = stream.cuda_stream
-
-    cfg = synth.CONFIGS["cfg1"]
-    k, n, q, g = cfg["k"], cfg["n"], cfg["q"], cfg["g"]
-    b_w, b_total = synth.algorithmic_bytes(k, n, q, g, False, 1)
-    w = synth.make_weight(k, n, q, g, seed=1)
-    x16 = synth.make_x(1, k, seed=1)
-
-    copies = max(1, args.copies)
-    weights = [lutgemm.BCQWeight(w["bW"], w["alpha"], k, n, q, k // g, None) for _ in range(copies)]
-    xd = torch.from_numpy(x16).to(dev)
-    yd = torch.zeros((copies, n), dtype=torch.float16, device=dev)
-    # launch plan: measured once on the first copy (a few untimed launches), same plan for all
-    plan = weights[0].autotune(sh)
-    for wgt in weights[1:]:
-        wgt.set_plan(plan["waves"], plan["k_splits"])
-
-    def sequence(count, rotate=True):
-        return lutgemm.MatvecSequence(
-            [(weights[(i % copies) if rotate else 0], xd.data_ptr(), yd[(i % copies) if rotate else 0].data_ptr(), 1)
-             for i in range(count)])
-
-    warm = sequence(max(1, args.warmup))
-    timed = sequence(args.steps)
-    hot = sequence(args.steps, rotate=False)
-
+    warm = lutgemm.MatvecSequence(pt.items(max(1, warmup)))
+    timed = lutgemm.MatvecSequence(pt.items(steps))
+    hot = lutgemm.MatvecSequence(pt.items(steps, rotate=False))
     warm.launch(sh)
     torch.cuda.synchronize()
     ms = event_time_ms(torch, lambda: timed.launch(sh), stream)
     torch.cuda.synchronize()
     ms_hot = event_time_ms(torch, lambda: hot.launch(sh), stream)
     torch.cuda.synchronize()
+    return ms * 1e3 / steps, ms_hot * 1e3 / steps
 
-    us = ms * 1e3 / args.steps
-    us_hot = ms_hot * 1e3 / args.steps
-    weight_gbs = b_w / (us * 1e-6) / 1e9
-    achieved = b_total / (us * 1e-6) / 1e9
 
-    # parity of what was just timed, against the double-precision oracle (checker only)
-    from oracle import oracle
-    truth = oracle.matvec_f64(w["bW"], w["alpha"].astype(np.float16), None, x16)
-    y = yd[0].cpu().numpy()
-    mean_abs, max_abs, rel_l2 = oracle.error_stats(y, truth)
-    ref_y = oracle.ref_kernel_fp16(w["bW"][:, :, :1024], w["alpha"].astype(np.float16)[:, :, :1024], None, x16[0])
-    ref_err = oracle.error_stats(ref_y, truth[0, :1024])
+def point_record(pt, us, us_hot):
+    return {"k": pt.k, "n": pt.n, "q": pt.q, "g": pt.g, "m": pt.m, "offset": pt.has_offset,
+            "us_per_matvec": us, "weight_GBps": pt.b_w / us / 1e3, "pct_hbm_peak": pt.b_w / us / 1e3 / HBM_PEAK_GBS * 100,
+            "hot_us_per_matvec": us_hot, "packed_weight_bytes": pt.b_w, "weight_copies_rotated": pt.copies,
+            "plan": pt.plan}
+
+
+def base_line(args, metric, value, us, workload, extra_config=None):
+    cfg = {"workload": workload}
+    cfg.update(extra_config or {})
+    return {
+        "metric": metric, "value": value, "unit": "GB/s (packed-weight bytes / matvec time)",
+        "us_per_matvec": us, "pct_hbm_peak": 100.0 * value / HBM_PEAK_GBS,
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": None,
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "fp16 in/out, fp32 accumulate",
+        "data": "synthetic (seeded; Bernoulli signs, |N(0,0.02)| scales, N(0,1) fp16 activations)",
+        "config": cfg,
+    }
+
+
+def run_single(args, lutgemm, synth, torch, dev, stream, name):
+    cfg = synth.CONFIGS[name]
+    k, n, q, g = cfg["k"], cfg["n"], cfg["q"], cfg["g"]
+    pt = Point(lutgemm, synth, torch, dev, k, n, q, g, cfg["rtn"], 1, 1, stream.cuda_stream,
+               copies=args.copies if name == "cfg1" else None)
+    us, us_hot = time_point(lutgemm, torch, stream, pt, args.steps, args.warmup)
+    weight_gbs = pt.b_w / (us * 1e-6) / 1e9
+    achieved = pt.b_total / (us * 1e-6) / 1e9
+    parity, truth = pt.parity(None if name != "cfg2" else 4096)
+
+    metric = METRIC if name == "cfg1" else "µs/matvec + weight-GB/s (%% HBM peak), k=%d n=%d q=%d g=%d m=1 fp16" % (k, n, q, g)
+    workload = "%s: BCQ matvec m=1 k=%d n=%d q=%d g=%d %s" % (
+        name, k, n, q, g, "RTN codes as BCQ with offset" if cfg["rtn"] else "no offset")
+    line = base_line(args, metric, weight_gbs, us, workload,
+                     {"weight_copies_rotated": pt.copies, "packed_weight_bytes": pt.b_w, "plan": pt.plan})
+    line["ms_per_step"] = us / 1e3
+    kernel = "lut_matvec_kernel<%d,%s,1>" % (q, "true" if pt.has_offset else "false")
+    line["roofline"] = {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                        "frac": achieved / HBM_PEAK_GBS,
+                        "traffic": CFG1_MEASURED_TRAFFIC_BYTES if name == "cfg1" else None,
+                        "kernel": kernel, "algorithmic_bytes_per_launch": pt.b_total, "avg_launch_us": us}
+    line["hot_single_copy"] = {"us_per_matvec": us_hot, "weight_GBps": pt.b_w / (us_hot * 1e-6) / 1e9}
+    if name == "cfg1":
+        import numpy as np
+        from oracle import oracle
+        ref_y = oracle.ref_kernel_fp16(pt.w["bW"][:, :, :1024], pt.w["alpha"].astype(np.float16)[:, :, :1024], None, pt.x16[0])
+        ref_err = oracle.error_stats(ref_y, truth[0, :1024])
+        parity["emulated_reference_kernel_first_1024_outputs"] = {
+            "mean_abs": ref_err[0], "max_abs": ref_err[1], "rel_l2": ref_err[2]}
+    line["parity"] = parity
 
     if args.copy_calibration:
         src = torch.empty(128 * 1024 * 1024, dtype=torch.float16, device=dev).fill_(1.0)  # 256 MiB
@@ -153,11 +225,11 @@ def main():
         del src, dst
 
     dense = None
-    if not args.no_dense:
+    if name == "cfg1" and not args.no_dense:
         # dense fp16 GEMV of the same shape through the vendor library (rocBLAS/hipBLASLt via torch)
         nd = 5  # 5 x 302 MB > 4 x last-level cache
         Wd = [torch.randn((n, k), dtype=torch.float16, device=dev) * 0.03 for _ in range(nd)]
-        xv = xd[0]
+        xv = pt.xd[0]
         outs = torch.empty((nd, n), dtype=torch.float16, device=dev)
         for i in range(10):
             torch.mv(Wd[i % nd], xv, out=outs[i % nd])
@@ -174,42 +246,160 @@ def main():
                  "GBps": (2 * k * n + 2 * k + 2 * n) / (dense_us * 1e-6) / 1e9,
                  "lut_speedup": dense_us / us}
         del Wd
+    line["dense_fp16_gemv"] = dense
+    line["cpu_baseline"] = None
+    if name == "cfg1" and not args.no_cpu:
+        line["cpu_baseline"] = cpu_baseline(synth, cfg, pt.x16, pt.w, truth)
+    pt.close()
+    return line
 
-    cpu = None
-    if not args.no_cpu:
-        cpu, ycpu = cpu_baseline(cfg, x16, w)
-        cpu["max_abs_vs_truth"] = float(np.abs(ycpu[0].astype(np.float64) - truth[0, :ycpu.shape[1]]).max())
 
-    line = {
-        "metric": METRIC,
-        "value": weight_gbs,
-        "unit": "GB/s (packed-weight bytes / matvec time)",
-        "us_per_matvec": us,
-        "pct_hbm_peak": 100.0 * weight_gbs / HBM_PEAK_GBS,
-        "n_gpus": 1,
-        "steps": args.steps,
-        "warmup": args.warmup,
-        "ms_per_step": ms / args.steps,
-        "higher_is_better": True,
-        "scaling": "weak",
-        "vs_baseline": None,
-        "dtype": "fp16 in/out, fp32 accumulate",
-        "data": "synthetic (seeded; Bernoulli signs, |N(0,0.02)| scales, N(0,1) fp16 activations)",
-        "config": {"workload": "cfg1: BCQ matvec m=1 k=12288 n=12288 q=3 g=128 no offset",
-                   "weight_copies_rotated": copies, "packed_weight_bytes": b_w,
-                   "plan": weights[0].plan()},
-        "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": achieved / HBM_PEAK_GBS, "traffic": None,
-                     "kernel": "lut_matvec_kernel<3,false,1>", "algorithmic_bytes_per_launch": b_total,
-                     "avg_launch_us": us},
-        "hot_single_copy": {"us_per_matvec": us_hot, "weight_GBps": b_w / (us_hot * 1e-6) / 1e9},
-        "parity": {"truth": "fp64 accumulation over fp16-rounded inputs (oracle)",
-                   "mean_abs": mean_abs, "max_abs": max_abs, "rel_l2": rel_l2,
-                   "emulated_reference_kernel_first_1024_outputs": {
-                       "mean_abs": ref_err[0], "max_abs": ref_err[1], "rel_l2": ref_err[2]}},
-        "dense_fp16_gemv": dense,
-        "cpu_baseline": cpu,
-    }
+def run_cfg3(args, lutgemm, synth, torch, dev, stream):
+    points = []
+    tot_bytes = tot_us = 0.0
+    worst = 0.0
+    for c in synth.CFG3_POINTS:
+        pt = Point(lutgemm, synth, torch, dev, c["k"], c["n"], c["q"], c["g"], False, 1, c["q"] * 10000 + c["g"],
+                   stream.cuda_stream)
+        us, us_hot = time_point(lutgemm, torch, stream, pt, args.steps, args.warmup)
+        rec = point_record(pt, us, us_hot)
+        rec["parity"], _ = pt.parity(2048)
+        worst = max(worst, rec["parity"]["max_abs"])
+        points.append(rec)
+        tot_bytes += pt.b_w
+        tot_us += us
+        pt.close()
+    value = tot_bytes / tot_us / 1e3
+    line = base_line(args, "weight-GB/s over the k=n=7168 sweep (q 1..4 x g 32,64,128,k), m=1 fp16", value,
+                     tot_us / len(points), "cfg3: 16 BCQ matvecs k=n=7168, q in 1..4, g in {32,64,128,7168}",
+                     {"points": len(points)})
+    line["ms_per_step"] = tot_us / 1e3
+    line["points"] = points
+    line["parity"] = {"worst_max_abs": worst, "outputs_checked_per_point": 2048}
+    line["roofline"] = {"bound": "hbm", "achieved": value, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                        "frac": value / HBM_PEAK_GBS, "traffic": None, "kernel": "lut_matvec_kernel<q,false,gsub>",
+                        "note": "aggregate packed-weight bytes / summed time over the 16 points"}
+    line["cpu_baseline"] = None
+    return line
+
+
+def run_cfg4(args, lutgemm, synth, torch, dev, stream):
+    """One decoder layer's four matvecs back to back (q=2, g=128): a step is the chain."""
+    m = args.m
+    sh = stream.cuda_stream
+    names = ["qkv", "out", "fc1", "fc2"]
+    pts = {}
+    step_bytes = sum(synth.algorithmic_bytes(L["k"], L["n"], 2, 128, False, m)[0] for L in synth.CFG4_LAYERS.values())
+    copies = max(2, int(math.ceil(4.0 * LLC_BYTES / step_bytes)) + 1)  # every launch misses the cache
+    for i, nm in enumerate(names):
+        L = synth.CFG4_LAYERS[nm]
+        pts[nm] = Point(lutgemm, synth, torch, dev, L["k"], L["n"], 2, 128, False, m, 400 + i, sh, copies=copies)
+    layers = []
+    for nm in names:
+        us, us_hot = time_point(lutgemm, torch, stream, pts[nm], args.steps, args.warmup)
+        rec = point_record(pts[nm], us, us_hot)
+        rec["layer"] = nm
+        rec["parity"], _ = pts[nm].parity(2048)
+        layers.append(rec)
+
+    def chain_items(steps):
+        out = []
+        for s in range(steps):
+            for nm in names:
+                out.extend(pts[nm].items(1, offset=s))
+        return out
+
+    warm = lutgemm.MatvecSequence(chain_items(max(1, args.warmup)))
+    timed = lutgemm.MatvecSequence(chain_items(args.steps))
+    warm.launch(sh)
+    torch.cuda.synchronize()
+    ms = event_time_ms(torch, lambda: timed.launch(sh), stream)
+    chain_us = ms * 1e3 / args.steps
+    graph = None
+    if args.graph:
+        # the same chain replayed from a captured HIP graph: one graph = `copies` steps, so that the
+        # rotation over weight copies is part of the graph; replays are checked against the eager result
+        eager = [pts[nm].yd.clone() for nm in names]
+        g = torch.cuda.CUDAGraph()
+        seq = lutgemm.MatvecSequence(chain_items(copies))
+        side = torch.cuda.Stream()
+        side.wait_stream(stream)
+        with torch.cuda.stream(side):
+            seq.launch(side.cuda_stream)  # warm-up on the capture stream
+            side.synchronize()
+            with torch.cuda.graph(g, stream=side):
+                seq.launch(torch.cuda.current_stream().cuda_stream)
+        stream.wait_stream(side)
+        torch.cuda.synchronize()
+        reps = max(1, args.steps // copies)
+        same = True
+        for _ in range(3):
+            for nm in names:
+                pts[nm].yd.zero_()
+            g.replay()
+            torch.cuda.synchronize()
+            same = same and all(torch.equal(pts[nm].yd, e) for nm, e in zip(names, eager))
+
+        def replay():
+            for _ in range(reps):
+                g.replay()
+        gms = event_time_ms(torch, replay, stream)
+        graph = {"us_per_layer_step": gms * 1e3 / (reps * copies), "steps_per_graph": copies,
+                 "replays_equal_eager": bool(same)}
+    value = step_bytes / chain_us / 1e3
+    line = base_line(args, "µs per decoder layer (QKV+out+FC1+FC2 matvecs) + weight-GB/s, q=2 g=128 m=%d fp16" % m,
+                     value, chain_us / 4.0, "cfg4: OPT-175B decoder layer matvecs q=2 g=128 m=%d" % m,
+                     {"weight_copies_rotated": copies, "packed_weight_bytes_per_step": step_bytes})
+    line["ms_per_step"] = chain_us / 1e3
+    line["us_per_layer_step"] = chain_us
+    line["sum_of_separately_timed_layers_us"] = sum(r["us_per_matvec"] for r in layers)
+    line["layers"] = layers
+    line["hip_graph"] = graph
+    line["roofline"] = {"bound": "hbm", "achieved": value, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                        "frac": value / HBM_PEAK_GBS, "traffic": None,
+                        "kernel": "lut_matvec_kernel<2,false,1>" if m == 1 else "lut_matvec2_kernel<2,false,1>",
+                        "note": "packed-weight bytes of the four layers / time of the chain"}
+    line["cpu_baseline"] = None
+    for p in pts.values():
+        p.close()
+    return line
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=400)
+    ap.add_argument("--warmup", type=int, default=2000,
+                    help="untimed steps first (the device reaches its sustained clocks only after some ms of load)")
+    ap.add_argument("--config", default="cfg1", choices=["cfg0", "cfg1", "cfg2", "cfg3", "cfg4"])
+    ap.add_argument("--m", type=int, default=1, help="activation rows (cfg4 only)")
+    ap.add_argument("--graph", action="store_true", help="cfg4: also replay the chain from a captured HIP graph")
+    ap.add_argument("--copies", type=int, default=17, help="cfg1: distinct weight copies rotated through")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-dense", action="store_true", help="skip the dense fp16 GEMV comparator")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="also run a plain 256 MiB device copy (known traffic) for scaling rocprof byte counters")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this build measures one GPU only (got --gpus %d); the path shards by output "
+                 "columns, see DESIGN.md" % args.gpus)
+
+    import torch
+
+    import lutgemm
+    from lutgemm import synth
+
+    lutgemm.load()  # no fallback: fails loudly if the HIP library is not built
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    stream = torch.cuda.current_stream()
+
+    if args.config == "cfg3":
+        line = run_cfg3(args, lutgemm, synth, torch, dev, stream)
+    elif args.config == "cfg4":
+        line = run_cfg4(args, lutgemm, synth, torch, dev, stream)
+    else:
+        line = run_single(args, lutgemm, synth, torch, dev, stream, args.config)
     print(json.dumps(line))
 
 

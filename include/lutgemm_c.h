@@ -130,8 +130,10 @@ int lutgemm_weight_set_plan(lutgemm_weight *w, int waves_per_group, int k_splits
 
 /* Measure the most promising launch plans on the device (a few launches each, on `stream`, with
  * scratch activations of its own) and keep the fastest.  Optional: the automatic plan is chosen
- * from a model, this replaces it by a measurement.  Synchronises `stream`; allocates and frees
- * temporary device buffers.  No counterpart in the reference, whose tile sizes are fixed
+ * from a model, this replaces it by a measurement.  The measurement streams the weight from
+ * HBM as a decoder does: it rotates over temporary device copies of the packed weight (about
+ * 1 GiB in total, at most 64 copies) so that no launch finds its weight in the memory-side
+ * cache.  Synchronises `stream`; allocates and frees temporary device buffers.  No counterpart in the reference, whose tile sizes are fixed
  * (lutGEMM/src/cuda/kernels/mv_fp16.hpp:122-124). */
 int lutgemm_weight_autotune(lutgemm_weight *w, void *stream);
 
