@@ -39,7 +39,7 @@ METRIC = "µs/matvec + weight-GB/s (% HBM peak), n=k=12288 q=3 g=128 m=1 fp16"
 # HBM bytes per cfg1 launch from the rocprofv3 counter runs summarised in
 # profiles/lut_matvec_kernel_cfg1.md (FETCH_SIZE and WRITE_SIZE, scaled by the factors a plain
 # copy kernel of known size reads on the same counters)
-CFG1_MEASURED_TRAFFIC_BYTES = 64.9e6
+CFG1_MEASURED_TRAFFIC_BYTES = 64.9e6  # plan 12 waves x 8 k-splits; 64.6e6 with 5 k-splits (fewer atomics)
 
 
 def event_time_ms(torch, fn, stream):
@@ -108,7 +108,7 @@ class Point:
     """One weight shape on the device: R rotating copies, an autotuned plan, buffers."""
 
     def __init__(self, lutgemm, synth, torch, dev, k, n, q, g, rtn, m, seed, stream_handle, copies=None,
-                 rotation_bytes=4 * LLC_BYTES):
+                 rotation_bytes=4 * LLC_BYTES, plan=None):
         self.k, self.n, self.q, self.g, self.m = k, n, q, g, m
         self.w = synth.make_weight(k, n, q, g, rtn=rtn, seed=seed)
         self.has_offset = self.w["q_bias"] is not None
@@ -117,7 +117,10 @@ class Point:
             copies = min(200, max(2, int(math.ceil(rotation_bytes / float(self.b_w))) + 1))
         self.copies = copies
         first = lutgemm.BCQWeight(self.w["bW"], self.w["alpha"], k, n, q, k // g, self.w["q_bias"])
-        first.autotune(stream_handle)  # measured once (a few untimed launches); clones keep the plan
+        if plan:
+            first.set_plan(plan[0], plan[1])
+        else:
+            first.autotune(stream_handle)  # measured once (untimed launches); clones keep the plan
         self.weights = [first] + [first.clone() for _ in range(copies - 1)]
         self.x16 = synth.make_x(m, k, seed=seed)
         self.xd = torch.from_numpy(self.x16).to(dev)
@@ -189,7 +192,7 @@ def run_single(args, lutgemm, synth, torch, dev, stream, name):
     cfg = synth.CONFIGS[name]
     k, n, q, g = cfg["k"], cfg["n"], cfg["q"], cfg["g"]
     pt = Point(lutgemm, synth, torch, dev, k, n, q, g, cfg["rtn"], 1, 1, stream.cuda_stream,
-               copies=args.copies if name == "cfg1" else None)
+               copies=args.copies if name == "cfg1" else None, plan=args.plan)
     us, us_hot = time_point(lutgemm, torch, stream, pt, args.steps, args.warmup)
     weight_gbs = pt.b_w / (us * 1e-6) / 1e9
     achieved = pt.b_total / (us * 1e-6) / 1e9
@@ -375,11 +378,15 @@ def main():
     ap.add_argument("--m", type=int, default=1, help="activation rows (cfg4 only)")
     ap.add_argument("--graph", action="store_true", help="cfg4: also replay the chain from a captured HIP graph")
     ap.add_argument("--copies", type=int, default=17, help="cfg1: distinct weight copies rotated through")
+    ap.add_argument("--plan", default=None,
+                    help="cfg0/1/2: WAVES,KSPLITS launch plan instead of the measured choice (profiling runs)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-dense", action="store_true", help="skip the dense fp16 GEMV comparator")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run a plain 256 MiB device copy (known traffic) for scaling rocprof byte counters")
     args = ap.parse_args()
+    if args.plan:
+        args.plan = tuple(int(v) for v in args.plan.split(","))
     if args.gpus != 1:
         sys.exit("bench.py: this build measures one GPU only (got --gpus %d); the path shards by output "
                  "columns, see DESIGN.md" % args.gpus)
