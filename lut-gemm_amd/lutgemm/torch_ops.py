@@ -1,0 +1,121 @@
+"""PyTorch-ROCm front end of the C ABI: a registered operator and a drop-in linear layer.
+
+  torch.ops.lutgemm.matvec(x, handle)   y[..., n] = x[..., k] @ W  for a packed BCQ weight
+  LutLinear                             nn.Module around one packed weight (+ optional bias)
+
+The operator launches on torch's current stream and allocates nothing but its output, so it can
+be captured into a HIP graph like any other torch op.  Batches larger than `dense_threshold`
+rows go through the dequantised fp16 weight and the library GEMM, the route the reference takes
+for every m > 1 (lutGEMM/src/kernels.cu:73-79); below it the LUT kernel streams the packed
+weight once per two rows.
+"""
+import weakref
+
+import numpy as np
+import torch
+
+from . import BCQWeight, LutGemmError, ERR_BAD_SHAPE, MAX_BATCH
+
+_weights = weakref.WeakValueDictionary()  # operator argument (an int) -> BCQWeight
+_next_id = [1]
+
+
+def register(weight):
+    """Make a BCQWeight addressable by the operator; returns its integer handle."""
+    hid = _next_id[0]
+    _next_id[0] += 1
+    _weights[hid] = weight
+    return hid
+
+
+def _lookup(handle):
+    w = _weights.get(int(handle))
+    if w is None:
+        raise LutGemmError(ERR_BAD_SHAPE, "operator handle %d is not registered (or its weight was freed)" % handle)
+    return w
+
+
+@torch.library.custom_op("lutgemm::matvec", mutates_args=())
+def matvec(x: torch.Tensor, handle: int) -> torch.Tensor:
+    w = _lookup(handle)
+    if not x.is_cuda or x.dtype != torch.float16:
+        raise TypeError("lutgemm::matvec needs a float16 tensor on the GPU, got %s on %s" % (x.dtype, x.device))
+    if x.shape[-1] != w.kSize:
+        raise LutGemmError(ERR_BAD_SHAPE, "last dimension %d != k %d" % (x.shape[-1], w.kSize))
+    x2 = x.reshape(-1, w.kSize).contiguous()
+    m = x2.shape[0]
+    y = torch.empty((m, w.mSize), dtype=torch.float16, device=x.device)
+    stream = torch.cuda.current_stream(x.device).cuda_stream
+    with torch.cuda.device(x.device):
+        for r0 in range(0, m, MAX_BATCH):
+            rows = min(MAX_BATCH, m - r0)
+            w.matvec(x2[r0:r0 + rows].data_ptr(), y[r0:r0 + rows].data_ptr(), rows, stream)
+    return y.reshape(x.shape[:-1] + (w.mSize,))
+
+
+@matvec.register_fake
+def _(x, handle):
+    w = _lookup(handle)
+    return x.new_empty(x.shape[:-1] + (w.mSize,))
+
+
+class LutLinear(torch.nn.Module):
+    """y = x @ W (+ bias) with W held as a packed BCQ weight on the current device.
+
+    container: dict(bW, alpha, q_bias, k, n, q, num_groups) as quantize.to_container returns.
+    """
+
+    def __init__(self, container, bias=None, dense_threshold=16, autotune=False):
+        super().__init__()
+        c = container
+        self.weight = BCQWeight(c["bW"], c["alpha"], c["k"], c["n"], c["q"], c["num_groups"], c.get("q_bias"))
+        if autotune:
+            self.weight.autotune(torch.cuda.current_stream().cuda_stream)
+        self.handle = register(self.weight)
+        self.in_features, self.out_features = c["k"], c["n"]
+        self.dense_threshold = dense_threshold
+        self._dense = None
+        if bias is not None:
+            self.register_buffer("bias", torch.as_tensor(bias).to(torch.float16).cuda())
+        else:
+            self.bias = None
+
+    @classmethod
+    def from_file(cls, path, bias=None, **kw):
+        self = cls.__new__(cls)
+        torch.nn.Module.__init__(self)
+        self.weight = BCQWeight.load(path)
+        self.handle = register(self.weight)
+        self.in_features, self.out_features = self.weight.kSize, self.weight.mSize
+        self.dense_threshold = kw.get("dense_threshold", 16)
+        self._dense = None
+        self.bias = None if bias is None else torch.as_tensor(bias).to(torch.float16).cuda()
+        return self
+
+    @classmethod
+    def from_linear(cls, linear, qbits, group_size=128, method="rtn", rounds=15, **kw):
+        """Quantise a torch.nn.Linear (weight [out, in]) and pack it."""
+        from . import quantize
+        c, _ = quantize.quantize_linear(linear.weight.detach().float(), qbits, group_size, method, rounds)
+        b = None if linear.bias is None else linear.bias.detach()
+        return cls(c, bias=b, **kw)
+
+    def dense_weight(self):
+        """Dequantised fp16 W [k][n] on the device (built once, kept for large batches)."""
+        if self._dense is None:
+            W = torch.empty((self.in_features, self.out_features), dtype=torch.float16, device="cuda")
+            self.weight.dequantize(W.data_ptr(), False, torch.cuda.current_stream().cuda_stream)
+            self._dense = W
+        return self._dense
+
+    def forward(self, x):
+        rows = x.numel() // x.shape[-1]
+        if rows > self.dense_threshold:
+            y = x.to(torch.float16) @ self.dense_weight()
+        else:
+            y = torch.ops.lutgemm.matvec(x, self.handle)
+        return y if self.bias is None else y + self.bias
+
+
+def container_from_numpy(bW, alpha, k, n, q, num_groups, q_bias=None):
+    return dict(bW=np.asarray(bW), alpha=np.asarray(alpha), q_bias=q_bias, k=k, n=n, q=q, num_groups=num_groups)

@@ -1,0 +1,96 @@
+"""The PyTorch operator and LutLinear on the GPU: parity with the oracle, the dense route for
+large batches, and replay from a captured HIP graph."""
+import numpy as np
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+
+def _layer(seed, out_f=320, in_f=1024, bias=True):
+    gen = torch.Generator().manual_seed(seed)
+    lin = torch.nn.Linear(in_f, out_f, bias=bias)
+    with torch.no_grad():
+        lin.weight.copy_(torch.randn(out_f, in_f, generator=gen) * 0.03)
+        if bias:
+            lin.bias.copy_(torch.randn(out_f, generator=gen) * 0.1)
+    return lin, gen
+
+
+@pytest.mark.parametrize("method,qbits", [("rtn", 4), ("bcq", 3)])
+def test_lut_linear_matches_oracle(lutgemm, oracle, device, method, qbits):
+    from gpu_util import assert_within_tolerance
+    from lutgemm import quantize, torch_ops
+    print("case LutLinear", method, qbits, flush=True)
+    lin, gen = _layer(1)
+    c, w_hat = quantize.quantize_linear(lin.weight.detach(), qbits, 128, method, rounds=5)
+    layer = torch_ops.LutLinear(c, bias=lin.bias.detach())
+    x = torch.randn(2, 3, 1024, generator=gen).to(torch.float16)
+    y = layer(x.to(device))
+    assert y.shape == (2, 3, 320) and y.dtype == torch.float16
+    a16 = c["alpha"].astype(np.float16)
+    z16 = c["q_bias"].astype(np.float16) if c["q_bias"] is not None else None
+    truth = oracle.matvec_f64(c["bW"], a16, z16, x.reshape(-1, 1024).numpy())
+    got = torch.ops.lutgemm.matvec(x.to(device), layer.handle).cpu().numpy().reshape(-1, 320)
+    assert_within_tolerance(got, truth, "operator")
+    want = truth + lin.bias.detach().to(torch.float16).double().numpy()
+    assert np.abs(y.cpu().double().numpy().reshape(-1, 320) - want).max() <= 2e-2
+
+
+def test_large_batches_take_the_dense_route(lutgemm, oracle, device):
+    from lutgemm import quantize, torch_ops
+    lin, gen = _layer(2, bias=False)
+    c, _ = quantize.quantize_linear(lin.weight.detach(), 4, 128, "rtn")
+    layer = torch_ops.LutLinear(c, dense_threshold=8)
+    x = torch.randn(40, 1024, generator=gen).to(torch.float16)
+    y_dense = layer(x.to(device))                       # 40 rows > threshold: dequantise + GEMM
+    assert layer._dense is not None and layer._dense.shape == (1024, 320)
+    y_lut = torch.ops.lutgemm.matvec(x.to(device), layer.handle)
+    # the dense weight is the oracle's dense weight rounded to fp16
+    a16 = c["alpha"].astype(np.float16)
+    z16 = c["q_bias"].astype(np.float16)
+    dense = oracle.dense_weight_f64(c["bW"], a16, z16)
+    assert np.array_equal(layer._dense.cpu().numpy(), dense.astype(np.float16))
+    truth = x.double().numpy() @ dense
+    assert np.abs(y_lut.cpu().double().numpy() - truth).max() <= 1e-2
+    assert np.abs(y_dense.cpu().double().numpy() - truth).max() <= 3e-2   # fp16 weight + library GEMM
+
+
+def test_operator_replays_from_a_hip_graph(lutgemm, device):
+    from lutgemm import quantize, torch_ops
+    lin, gen = _layer(3, bias=False)
+    c, _ = quantize.quantize_linear(lin.weight.detach(), 3, 128, "bcq", rounds=2)
+    layer = torch_ops.LutLinear(c)
+    xs = [torch.randn(2, 1024, generator=gen).to(torch.float16).to(device) for _ in range(3)]
+    eager = [layer(x).clone() for x in xs]
+    static_x = xs[0].clone()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        layer(static_x)
+        side.synchronize()
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g, stream=side):
+            static_y = layer(static_x)
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    for rep in range(2):
+        for x, want in zip(xs, eager):
+            static_x.copy_(x)
+            torch.cuda.synchronize()
+            g.replay()
+            torch.cuda.synchronize()
+            assert torch.equal(static_y, want), "replay %d differs from the eager result" % rep
+
+
+def test_operator_argument_checks(lutgemm, device):
+    from lutgemm import quantize, torch_ops
+    lin, _ = _layer(4, bias=False)
+    c, _ = quantize.quantize_linear(lin.weight.detach(), 2, 128, "rtn")
+    layer = torch_ops.LutLinear(c)
+    with pytest.raises(Exception):
+        torch.ops.lutgemm.matvec(torch.zeros(1, 1024, dtype=torch.float32, device=device), layer.handle)
+    with pytest.raises(Exception):
+        torch.ops.lutgemm.matvec(torch.zeros(1, 512, dtype=torch.float16, device=device), layer.handle)
+    with pytest.raises(Exception):
+        torch.ops.lutgemm.matvec(torch.zeros(1, 1024, dtype=torch.float16, device=device), 10 ** 9)
