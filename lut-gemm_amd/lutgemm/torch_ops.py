@@ -65,7 +65,7 @@ class LutLinear(torch.nn.Module):
     container: dict(bW, alpha, q_bias, k, n, q, num_groups) as quantize.to_container returns.
     """
 
-    def __init__(self, container, bias=None, dense_threshold=16, autotune=False):
+    def __init__(self, container, bias=None, dense_threshold=7, autotune=False):
         super().__init__()
         c = container
         self.weight = BCQWeight(c["bW"], c["alpha"], c["k"], c["n"], c["q"], c["num_groups"], c.get("q_bias"))
@@ -87,7 +87,7 @@ class LutLinear(torch.nn.Module):
         self.weight = BCQWeight.load(path)
         self.handle = register(self.weight)
         self.in_features, self.out_features = self.weight.kSize, self.weight.mSize
-        self.dense_threshold = kw.get("dense_threshold", 16)
+        self.dense_threshold = kw.get("dense_threshold", 7)
         self._dense = None
         self.bias = None if bias is None else torch.as_tensor(bias).to(torch.float16).cuda()
         return self

@@ -140,9 +140,10 @@ def test_batched_rows_and_columns(lutgemm, oracle, device, m):
     (2560, 513, 4, 32, False), (96, 33, 4, 96, True), (7168, 224, 3, 128, True), (640, 70, 8, 128, False),
 ])
 def test_row_pairs_equal_single_rows_bit_for_bit(lutgemm, oracle, device, k, n, q, g, offset):
-    """Rows are processed two per pass over the weight; every row must come out exactly as a
-    one-row launch with the same plan produces it (same tables, same order of accumulation),
-    for every scale layout (g % 128, % 64, % 32), with and without offset, for several plans."""
+    """Rows go through the weight two per pass (a last single row if m is odd); each must come
+    out exactly as a one-row launch with the same plan produces it (same tables, same order of
+    accumulation), for every scale layout (g % 128, % 64, % 32), with and without offset, for
+    several plans."""
     from lutgemm import synth
     m = 5
     w, W = make(lutgemm, synth, k, n, q, g, offset=offset, seed=k + q)
@@ -156,6 +157,29 @@ def test_row_pairs_equal_single_rows_bit_for_bit(lutgemm, oracle, device, k, n, 
         for r in range(m):
             y1 = run_matvec(lutgemm, W, x[r:r + 1], device)
             assert np.array_equal(y[r].view(np.uint16), y1[0].view(np.uint16)), "row %d plan %s" % (r, W.plan())
+    W.close()
+
+
+@pytest.mark.parametrize("k,n,q,g,offset", [
+    (1536, 100, 2, 32, True), (1024, 96, 1, 64, False), (3072, 1000, 3, 64, True), (4096, 520, 3, 128, False),
+    (2560, 513, 4, 32, False), (96, 33, 4, 96, True), (7168, 224, 3, 128, True), (640, 70, 8, 128, False),
+    (512, 64, 8, 32, True), (12288, 256, 2, 128, False),
+])
+def test_many_rows(lutgemm, oracle, device, k, n, q, g, offset):
+    """Row counts that end in a two-row and in a one-row pass: every scale layout, with and
+    without offset, several plans; deterministic; row- and column-batched forms agree."""
+    from lutgemm import synth
+    w, W = make(lutgemm, synth, k, n, q, g, offset=offset, seed=k + 3 * q)
+    for m, (waves, ks) in zip((3, 4, 5, 6, 7, 8, 11), ((0, 0), (1, 1), (5, 2), (12, 3), (8, 2), (3, 4), (0, 0))):
+        say("case many rows", k, n, q, g, offset, m, waves, ks)
+        x = synth.make_x(m, k, seed=n + m)
+        truth = truth_of(oracle, w, x)
+        W.set_plan(waves, min(ks, (k + 511) // 512))
+        y = run_matvec(lutgemm, W, x, device)
+        assert_within_tolerance(y, truth, "m=%d plan=%s" % (m, W.plan()))
+        assert np.array_equal(y.view(np.uint16), run_matvec(lutgemm, W, x, device).view(np.uint16))
+        yc = run_matvec(lutgemm, W, x, device, cols=True)
+        assert np.array_equal(y.view(np.uint16), yc.view(np.uint16))
     W.close()
 
 
