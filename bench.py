@@ -388,8 +388,8 @@ def main():
     if args.plan:
         args.plan = tuple(int(v) for v in args.plan.split(","))
     if args.gpus != 1:
-        sys.exit("bench.py: this build measures one GPU only (got --gpus %d); the path shards by output "
-                 "columns, see DESIGN.md" % args.gpus)
+        sys.exit("bench.py: this build measures one GPU only (got --gpus %d); a matvec shards by output "
+                 "columns, no multi-GPU path is built" % args.gpus)
 
     import torch
 

@@ -88,8 +88,11 @@ double plan_cost(const Shape &s, int cus, int waves, int splits, Plan *out)
     const int ks = div_up(s.ts, bps);
     if (ks != splits) return -1.0;  // same plan as a smaller `splits`
     const long wgs = (long)ntiles * ks;
-    const double rounds = (double)((wgs + cus - 1) / cus);
-    const double active = (double)(wgs < cus ? wgs : cus);
+    // a workgroup with a single k-block needs one table set only: two of them share a compute
+    // unit (LDS and, up to 8 wavefronts each, registers allow it)
+    const long slots = (bps == 1 && waves <= 8) ? 2L * cus : (long)cus;
+    const double rounds = (double)((wgs + slots - 1) / slots);
+    const double active = (double)(wgs < slots ? wgs : slots);
     double bw = kFairBytes * cus / active;
     if (bw > kPeakBytes) bw = kPeakBytes;
     // a tile is requested one k-block ahead, so a k-block cannot take less than one memory

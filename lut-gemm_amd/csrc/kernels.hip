@@ -526,7 +526,9 @@ __global__ __launch_bounds__(768) void lut_matvec_kernel(MatvecArgs a)
 {
     constexpr int QO = Q + (OFF ? 1 : 0);
     // Two table sets: while the lookups of k-block t read one, the other is rebuilt for t+1.
-    __shared__ float table[2 * kTableFloats];
+    // Dynamic LDS: a workgroup with a single k-block is launched with one set only (64 KiB), so
+    // that two such workgroups fit a compute unit.
+    extern __shared__ float table[];
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -760,7 +762,14 @@ hipError_t launch_one(const MatvecArgs &a, int workgroups, int threads, hipStrea
     if (a.rows > 1)
         hipLaunchKernelGGL((lut_matvec2_kernel<Q, OFF, GSUB>), dim3(workgroups), dim3(threads), 0, stream, a);
     else
-        hipLaunchKernelGGL((lut_matvec_kernel<Q, OFF, GSUB>), dim3(workgroups), dim3(threads), 0, stream, a);
+    {
+        static const hipError_t attr = hipFuncSetAttribute(
+            reinterpret_cast<const void *>(&lut_matvec_kernel<Q, OFF, GSUB>),
+            hipFuncAttributeMaxDynamicSharedMemorySize, 2 * kTableFloats * (int)sizeof(float));
+        if (attr != hipSuccess) return attr;
+        const size_t lds = (size_t)(a.blocks_per_split == 1 ? 1 : 2) * kTableFloats * sizeof(float);
+        hipLaunchKernelGGL((lut_matvec_kernel<Q, OFF, GSUB>), dim3(workgroups), dim3(threads), lds, stream, a);
+    }
     return hipGetLastError();
 }
 

@@ -108,6 +108,33 @@ def test_command_line_packer(lutgemm, tmp_path):
     assert r.returncode != 0 and "not a packed-weight file" in r.stderr
 
 
+def test_file_entry_points_check_their_arguments(lutgemm, tmp_path):
+    """No device needed: null pointers and unreadable files are reported before any device work; a
+    good file on a machine without a GPU fails with the no-device status, not with a crash."""
+    import ctypes
+    import torch
+    from lutgemm import synth
+    L = lutgemm.load()
+    h = ctypes.c_void_p()
+    assert L.lutgemm_weight_load(None, ctypes.byref(h)) == lutgemm.ERR_NULL_POINTER
+    assert L.lutgemm_weight_load(b"/nonexistent/x.lutw", None) == lutgemm.ERR_NULL_POINTER
+    assert L.lutgemm_weight_load(b"/nonexistent/x.lutw", ctypes.byref(h)) == lutgemm.ERR_IO
+    assert b"cannot open" in L.lutgemm_last_error()
+    assert L.lutgemm_weight_save(None, b"/tmp/x.lutw") == lutgemm.ERR_NULL_POINTER
+    assert L.lutgemm_weight_clone(None, ctypes.byref(h)) == lutgemm.ERR_NULL_POINTER
+    assert L.lutgemm_pack_file(None, None, None, 512, 8, 1, 1, b"/tmp/x.lutw") == lutgemm.ERR_NULL_POINTER
+    assert L.lutgemm_unpack_file(None, None, None, None, None) == lutgemm.ERR_NULL_POINTER
+    assert L.lutgemm_status_string(lutgemm.ERR_IO) == b"file input/output failed"
+    assert h.value is None
+    if not torch.cuda.is_available():
+        w = problem(synth, 512, 40, 2, 128, False)
+        path = tmp_path / "w.lutw"
+        lutgemm.pack_file(path, w["bW"], w["alpha"], 512, 40, 2, 4, None)
+        with pytest.raises(lutgemm.LutGemmError) as e:
+            lutgemm.BCQWeight.load(path)
+        assert e.value.status == lutgemm.ERR_NO_DEVICE
+
+
 @pytest.mark.gpu
 @pytest.mark.parametrize("k,n,q,g,offset", [(2048, 300, 3, 128, True), (1536, 100, 2, 32, False)])
 def test_save_load_clone_on_device(lutgemm, oracle, device, tmp_path, k, n, q, g, offset):
