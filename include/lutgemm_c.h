@@ -86,7 +86,8 @@ int lutgemm_weight_info(const lutgemm_weight *w, lutgemm_weight_info_t *info);
  * Replaces lutGEMM::matmul(void* output, void* input, nQWeight_fp16&, int m, int algo)
  * (lutGEMM/include/kernels.h:27, lutGEMM/src/kernels.cu:64-71), which for m == 1 runs
  * kernel::nqmv (mv_fp16.hpp:121) or kernel::nqmv_bias (mv_fp16_bias.hpp:143); here every
- * 1 <= m <= LUTGEMM_MAX_BATCH stays on the table-lookup kernel.
+ * 1 <= m <= LUTGEMM_MAX_BATCH stays on the table-lookup kernels: rows go through the weight two
+ * per pass (one for a last odd row), every row bit-identical to its own one-row call.
  * Calls that overlap in time on the same handle race on its split-k accumulators. */
 #define LUTGEMM_MAX_BATCH 4096
 int lutgemm_matvec(const lutgemm_weight *w, const void *x, void *y, int m, void *stream);
