@@ -29,13 +29,19 @@ def _groups(w, group_size):
     return out_ch, in_ch, g
 
 
+def _uniform(x, scale, zero, maxq):
+    return scale * (torch.clamp(torch.round(x / scale) + zero, 0, maxq) - zero)
+
+
 @torch.no_grad()
-def rtn_quantize(w, qbits, group_size=-1, sym=False):
+def rtn_quantize(w, qbits, group_size=-1, sym=False, mse=False, norm=2.4, grid=100, maxshrink=0.8):
     """Uniform quantisation with one (scale, zero) per group of `group_size` input channels.
 
     Returns (scale [out, G, 1], zero [out, G, 1], codes int32 [out, G, g]) with
     w ~= scale * (codes - zero), codes in 0 .. 2^qbits - 1.  The range of a group always includes
-    zero; sym=True makes it symmetric about zero.
+    zero; sym=True makes it symmetric about zero.  mse=True shrinks the range of each group in
+    `grid` steps down to (1 - maxshrink) of it and keeps the (scale, zero) with the smallest
+    sum |error|^norm (the search of examples/utils.py:91-110).
     """
     out_ch, in_ch, g = _groups(w, group_size)
     maxq = float(2 ** qbits - 1)
@@ -51,6 +57,18 @@ def rtn_quantize(w, qbits, group_size=-1, sym=False):
     xmax = torch.where(flat, torch.full_like(xmax, 1.0), xmax)
     scale = (xmax - xmin) / maxq
     zero = torch.full_like(scale, (maxq + 1) / 2) if sym else torch.round(-xmin / scale)
+    if mse:
+        best = torch.full_like(scale, float("inf"))
+        full_zero = zero.clone()
+        for i in range(int(maxshrink * grid)):
+            p = 1.0 - i / grid
+            scale1 = p * (xmax - xmin) / maxq
+            zero1 = full_zero if sym else torch.round(-(p * xmin) / scale1)
+            err = (_uniform(x, scale1[:, None], zero1[:, None], maxq) - x).abs().pow(norm).sum(dim=1)
+            better = err < best
+            best = torch.where(better, err, best)
+            scale = torch.where(better, scale1, scale)
+            zero = torch.where(better, zero1, zero)
     codes = torch.clamp(torch.round(x / scale[:, None]) + zero[:, None], 0, maxq).to(torch.int32)
     G = in_ch // g
     return scale.reshape(out_ch, G, 1), zero.reshape(out_ch, G, 1), codes.reshape(out_ch, G, g)

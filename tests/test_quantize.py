@@ -37,6 +37,24 @@ def test_rtn_error_bound_and_range(qbits, g, sym):
         assert torch.all(zero == 2 ** qbits / 2)
 
 
+@pytest.mark.parametrize("qbits,sym", [(3, False), (4, False), (4, True)])
+def test_rtn_range_search_never_worse_in_its_own_norm(qbits, sym):
+    """mse=True tries the full range first (shrink factor 1), so per group its sum |error|^norm
+    cannot exceed the plain min/max result; with outliers stretching the range it is better overall."""
+    gen = torch.Generator().manual_seed(17)
+    w = torch.randn(32, 256, generator=gen) * 0.02
+    w[:, ::64] *= 8.0                                   # outliers that stretch the min/max range
+    plain = Q.rtn_quantize(w, qbits, 128, sym=sym)
+    tuned = Q.rtn_quantize(w, qbits, 128, sym=sym, mse=True)
+    def err(r):
+        return (Q.rtn_dequantize(*r) - w).reshape(32, 2, 128).abs().pow(2.4).sum(-1)
+    e0, e1 = err(plain), err(tuned)
+    assert torch.all(e1 <= e0 * (1 + 1e-6))
+    assert e1.sum() < e0.sum() * 0.97 and (e1 < e0 * 0.95).any()
+    assert tuned[2].min() >= 0 and tuned[2].max() <= 2 ** qbits - 1
+    assert torch.all(tuned[0] <= plain[0] * (1 + 1e-6))  # the range only shrinks
+
+
 @pytest.mark.parametrize("qbits", [1, 2, 3, 4, 8])
 def test_rtn_to_bcq_identity_over_all_codes(qbits):
     # every code value, several (scale, zero): sum_i alpha_i s_i + offset == scale (c - zero)
