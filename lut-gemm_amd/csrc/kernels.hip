@@ -18,6 +18,8 @@
 //    add their partials into a per-output fixed-point integer with one 64-bit atomic; the
 //    last arrival finishes the output.  Integer sums do not depend on arrival order, so the
 //    result is deterministic, and no memset or floating-point atomic on y is needed.
+//  * Batches take two activation rows per pass over the weight (lut_matvec2_kernel: table
+//    entries hold both rows, one 8-byte LDS read per lookup).
 #include <hip/hip_fp16.h>
 #include <hip/hip_runtime.h>
 
