@@ -23,6 +23,7 @@
 #include <hip/hip_fp16.h>
 #include <hip/hip_runtime.h>
 
+#include <atomic>
 #include <type_traits>
 #include <utility>
 
@@ -765,10 +766,19 @@ hipError_t launch_one(const MatvecArgs &a, int workgroups, int threads, hipStrea
         hipLaunchKernelGGL((lut_matvec2_kernel<Q, OFF, GSUB>), dim3(workgroups), dim3(threads), 0, stream, a);
     else
     {
-        static const hipError_t attr = hipFuncSetAttribute(
-            reinterpret_cast<const void *>(&lut_matvec_kernel<Q, OFF, GSUB>),
-            hipFuncAttributeMaxDynamicSharedMemorySize, 2 * kTableFloats * (int)sizeof(float));
-        if (attr != hipSuccess) return attr;
+        // more than 64 KiB of dynamic LDS has to be allowed once per kernel and device
+        static std::atomic<unsigned long long> allowed{0};
+        int dev = 0;
+        hipError_t e = hipGetDevice(&dev);
+        if (e != hipSuccess) return e;
+        const unsigned long long bit = 1ull << (dev & 63);
+        if (!(allowed.load(std::memory_order_relaxed) & bit)) {
+            e = hipFuncSetAttribute(reinterpret_cast<const void *>(&lut_matvec_kernel<Q, OFF, GSUB>),
+                                    hipFuncAttributeMaxDynamicSharedMemorySize,
+                                    2 * kTableFloats * (int)sizeof(float));
+            if (e != hipSuccess) return e;
+            allowed.fetch_or(bit, std::memory_order_relaxed);
+        }
         const size_t lds = (size_t)(a.blocks_per_split == 1 ? 1 : 2) * kTableFloats * sizeof(float);
         hipLaunchKernelGGL((lut_matvec_kernel<Q, OFF, GSUB>), dim3(workgroups), dim3(threads), lds, stream, a);
     }
