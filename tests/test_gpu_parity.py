@@ -260,3 +260,30 @@ def test_device_round_trip_and_dequantize(lutgemm, oracle, device):
                                         w["q_bias"].astype(np.float16) if off else None)
         assert np.all(np.abs(got.astype(np.float64) - dense) <= 2.0 ** -11 * np.abs(dense) + 2.0 ** -24)
         W.close()
+
+
+def test_random_shapes_plans_and_batches(lutgemm, oracle, device):
+    """Sixty seeded random problems: ragged k (any multiple of 32, so the last k-block and the
+    last scale group are partial), odd n, every q, group sizes with all three scale layouts,
+    with / without offset, 1..6 rows, random launch plans."""
+    from lutgemm import synth
+    rng = np.random.default_rng(20240607)
+    for case in range(60):
+        q = int(rng.integers(1, 9))
+        g = int(rng.choice([32, 64, 96, 128, 256, 384]))
+        G = int(rng.integers(1, 24))
+        k = g * G
+        n = int(rng.integers(1, 700))
+        offset = bool(rng.integers(0, 2))
+        m = int(rng.integers(1, 7))
+        ts = (k + 511) // 512
+        waves = int(rng.integers(0, 13))
+        ks = int(rng.integers(0, ts + 1))
+        say("case random", case, k, n, q, g, offset, m, waves, ks)
+        w, W = make(lutgemm, synth, k, n, q, g, offset=offset, seed=1000 + case)
+        W.set_plan(waves, ks)
+        x = synth.make_x(m, k, seed=case)
+        y = run_matvec(lutgemm, W, x, device, cols=bool(case % 2))
+        assert_within_tolerance(y, truth_of(oracle, w, x),
+                                "case %d k=%d n=%d q=%d g=%d off=%s m=%d plan=%s" % (case, k, n, q, g, offset, m, W.plan()))
+        W.close()
