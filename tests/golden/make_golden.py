@@ -4,7 +4,9 @@ The reference holds no data files or known-answer vectors for this path, and non
 imported or run here: inputs come from the seeded generator of this repository and the expected
 outputs from the CPU oracle (double-precision truth) after the oracle itself has been pinned by
 tests/test_oracle.py.  The fixtures freeze those answers so that a later change to the oracle, the
-generator or the library shows up as a diff against committed data.
+generator or the library shows up as a diff against committed data.  Beside every .npz lies the
+packed-weight file (.lutw) the host packer writes for it: a change of the tile layout or of the
+file format shows up the same way.
 
     python tests/golden/make_golden.py
 """
@@ -39,6 +41,9 @@ def main():
         np.savez_compressed(os.path.join(HERE, name + ".npz"), bW=w["bW"], alpha=w["alpha"].astype(np.float16),
                             q_bias=(z if z is not None else np.zeros(0, np.float16)), x=x, y=y,
                             meta=np.array([k, n, q, g, int(off), m]))
+        # the packed-weight file of the same problem: freezes the tile layout and the file format
+        import lutgemm
+        lutgemm.pack_file(os.path.join(HERE, name + ".lutw"), w["bW"], w["alpha"], k, n, q, k // g, w["q_bias"])
         print(name, y.shape, float(np.abs(y).max()))
 
 
