@@ -113,6 +113,31 @@ public:
 
     lutgemm_weight *handle() const { return handle_; }
 
+    // ---- additions without counterpart in the reference ----
+    // Write the packed weight to a file / replace this object's weight by a packed file's
+    // (no packing work on load).  A loaded weight is column-wise (is_row_wise_quantize = false).
+    void save(const char *path) const { detail::check(lutgemm_weight_save(handle_, path), "nQWeight_fp16::save"); }
+    void load(const char *path)
+    {
+        release();
+        detail::check(lutgemm_weight_load(path, &handle_), "nQWeight_fp16::load");
+        lutgemm_weight_info_t info;
+        detail::check(lutgemm_weight_info(handle_, &info), "nQWeight_fp16::load");
+        is_row_wise_quantize = false;
+        kSize = info.k;
+        mSize = info.n;
+        nb = info.q;
+        num_groups = info.num_groups;
+        group_size = info.group_size;
+        void *s = nullptr, *a = nullptr, *z = nullptr;
+        detail::check(lutgemm_weight_device_ptrs(handle_, &s, &a, &z), "nQWeight_fp16::load");
+        bWeight = static_cast<unsigned int *>(s);
+        alpha = a;
+        q_bias = z;
+    }
+    // Measure launch plans on the device and keep the fastest (the default plan comes from a model).
+    void autotune() { detail::check(lutgemm_weight_autotune(handle_, nullptr), "nQWeight_fp16::autotune"); }
+
 private:
     void release()
     {

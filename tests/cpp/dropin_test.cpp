@@ -185,6 +185,26 @@ int main(int argc, char **argv)
             }
         printf("getDequantiedWeight / dequantize_cpu: %d wrong weights\n", wbad);
         bad += wbad;
+        // additions to the container: packed file round trip and measured plan keep the results
+        {
+            const char *path = "/tmp/lutgemm_dropin_test.lutw";
+            nqW.save(path);
+            lutGEMM::nQWeight_fp16 loaded;
+            loaded.load(path);
+            loaded.autotune();
+            std::remove(path);
+            int ldiff = loaded.kSize != K || loaded.mSize != N || loaded.nb != q || loaded.num_groups != K / g;
+            lutGEMM::matmul((void *)dy, (void *)dxr, loaded, n);
+            HIP_OK(hipDeviceSynchronize());
+            std::vector<_Float16> y2((size_t)n * N);
+            HIP_OK(hipMemcpy(y2.data(), dy, y2.size() * 2, hipMemcpyDeviceToHost));
+            // another plan changes the summation order only: unit scales and these activations leave
+            // the results within one fp16 step
+            for (size_t i = 0; i < y2.size(); i++)
+                ldiff += std::fabs((float)y2[i] - (float)y_rows[i]) > 4e-3f * std::fmax(1.f, std::fabs((float)y_rows[i]));
+            printf("save / load / autotune: %d differing outputs\n", ldiff);
+            bad += ldiff;
+        }
         HIP_OK(hipFree(dx)); HIP_OK(hipFree(dxr)); HIP_OK(hipFree(dy)); HIP_OK(hipFree(dyr));
     }
     {
