@@ -31,7 +31,7 @@ typedef enum lutgemm_status {
     LUTGEMM_OK = 0,
     LUTGEMM_ERR_NULL_POINTER = 1,  /* a required pointer argument is NULL */
     LUTGEMM_ERR_BAD_SHAPE = 2,     /* k, n, q, num_groups or m violate the preconditions */
-    LUTGEMM_ERR_NO_DEVICE = 3,     /* no HIP device / the device is not usable */
+    LUTGEMM_ERR_NO_DEVICE = 3,     /* no HIP device, or the current device is not the handle's */
     LUTGEMM_ERR_HIP = 4,           /* a HIP runtime call failed; see lutgemm_last_error() */
     LUTGEMM_ERR_OUT_OF_MEMORY = 5, /* host or device allocation failed */
     LUTGEMM_ERR_UNSUPPORTED = 6,   /* valid request outside what this build implements */

@@ -116,6 +116,17 @@ Plan choose_plan(const Shape &s, int cus)
     return best;
 }
 
+// A handle's device memory belongs to the device that was current when it was created.
+int check_device(const lutgemm_weight *w)
+{
+    int dev = -1;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return hip_fail(e, "hipGetDevice");
+    if (dev != w->device)
+        return fail(LUTGEMM_ERR_NO_DEVICE, "the weight lives on device %d but device %d is current", w->device, dev);
+    return LUTGEMM_OK;
+}
+
 int alloc_workspace(lutgemm_weight *w)
 {
     if (w->d_accum) return LUTGEMM_OK;  // size depends on the shape only
@@ -301,6 +312,7 @@ int run_matvec(const lutgemm_weight *w, const void *x, void *y, int m, void *str
     if (!w || !x || !y) return fail(LUTGEMM_ERR_NULL_POINTER, "null argument to matvec");
     if (m < 1 || m > LUTGEMM_MAX_BATCH)
         return fail(LUTGEMM_ERR_BAD_SHAPE, "m=%d outside 1..%d", m, LUTGEMM_MAX_BATCH);
+    if (int st_dev = check_device(w)) return st_dev;
     const Shape &s = w->shape;
     lutgemm_kernels::MatvecArgs a{};
     a.signs = w->d_signs;
@@ -506,6 +518,7 @@ int lutgemm_matvec_many(const lutgemm_weight *const *ws, const void *const *xs, 
 int lutgemm_dequantize(const lutgemm_weight *w, void *d_fW, int transposed, void *stream)
 {
     if (!w || !d_fW) return fail(LUTGEMM_ERR_NULL_POINTER, "null argument to dequantize");
+    if (int st_dev = check_device(w)) return st_dev;
     const Shape &s = w->shape;
     lutgemm_kernels::DequantArgs a{};
     a.signs = w->d_signs;
