@@ -88,7 +88,11 @@ int lutgemm_weight_info(const lutgemm_weight *w, lutgemm_weight_info_t *info);
  * kernel::nqmv (mv_fp16.hpp:121) or kernel::nqmv_bias (mv_fp16_bias.hpp:143); here every
  * 1 <= m <= LUTGEMM_MAX_BATCH stays on the table-lookup kernels: rows go through the weight two
  * per pass (one for a last odd row), every row bit-identical to its own one-row call.
- * Calls that overlap in time on the same handle race on its split-k accumulators. */
+ * Calls that overlap in time on the same handle race on its split-k accumulators.
+ * Finite inputs are assumed: with more than one k-split the partial sums are added as fixed-point
+ * integers (2^-24 resolution, saturating at about +-8.4e6, far beyond binary16's range), so an
+ * infinite partial sum still yields an infinity of that sign, but a NaN one yields an infinity
+ * instead of a NaN. */
 #define LUTGEMM_MAX_BATCH 4096
 int lutgemm_matvec(const lutgemm_weight *w, const void *x, void *y, int m, void *stream);
 
