@@ -287,3 +287,32 @@ def test_random_shapes_plans_and_batches(lutgemm, oracle, device):
         assert_within_tolerance(y, truth_of(oracle, w, x),
                                 "case %d k=%d n=%d q=%d g=%d off=%s m=%d plan=%s" % (case, k, n, q, g, offset, m, W.plan()))
         W.close()
+
+
+def test_non_finite_activations(lutgemm, device):
+    """Documented behaviour: without k-splits IEEE arithmetic propagates (NaN stays NaN); with
+    k-splits an infinite partial sum gives an infinity of its sign and a NaN one an infinity; all
+    outputs stay finite where the activations are, and the split-k words return to zero."""
+    from lutgemm import synth
+    k, n, q, g = 2048, 96, 2, 128
+    w, W = make(lutgemm, synth, k, n, q, g, seed=3)
+    x = synth.make_x(1, k, seed=3)
+    good = None
+    for ks in (1, 4):
+        W.set_plan(2, ks)
+        clean = run_matvec(lutgemm, W, x, device)
+        assert np.isfinite(clean).all()
+        good = clean if good is None else good
+        xn = x.copy()
+        xn[0, 700] = np.nan
+        yn = run_matvec(lutgemm, W, xn, device)
+        assert (np.isnan(yn).all() if ks == 1 else np.isinf(yn).all()), ks
+        xi = x.copy()
+        xi[0, 5] = np.inf
+        yi = run_matvec(lutgemm, W, xi, device)
+        assert not np.isfinite(yi).any()
+        # the handle is as good as new afterwards
+        again = run_matvec(lutgemm, W, x, device)
+        assert np.array_equal(again.view(np.uint16), clean.view(np.uint16))
+    W.close()
+
