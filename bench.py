@@ -210,6 +210,20 @@ def run_single(args, lutgemm, synth, torch, dev, stream, name):
                         "traffic": CFG1_MEASURED_TRAFFIC_BYTES if name == "cfg1" else None,
                         "kernel": kernel, "algorithmic_bytes_per_launch": pt.b_total, "avg_launch_us": us}
     line["hot_single_copy"] = {"us_per_matvec": us_hot, "weight_GBps": pt.b_w / (us_hot * 1e-6) / 1e9}
+    # the device's pure-read time for the same tiles, same grid, same rotation over the copies
+    lutgemm.read_probe(pt.weights * 3, stream.cuda_stream)
+    torch.cuda.synchronize()
+    reads = max(1, args.steps)
+    order = [pt.weights[i % pt.copies] for i in range(reads)]
+
+    def run_reads():
+        lutgemm.read_probe(order, stream.cuda_stream)
+    rms = event_time_ms(torch, run_reads, stream)
+    read_us = rms * 1e3 / reads
+    info = pt.weights[0].info()
+    tile_bytes = info.device_bytes - 8 * 2 * 32 * ((n + 31) // 32)  # packed tiles incl. padding, without the split-k words
+    line["pure_read_same_tiles"] = {"us": read_us, "bytes": tile_bytes, "GBps": tile_bytes / read_us / 1e3,
+                                    "matvec_time_over_read_time": us / read_us}
     if name == "cfg1":
         import numpy as np
         from oracle import oracle

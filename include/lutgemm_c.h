@@ -118,6 +118,13 @@ int lutgemm_matvec_many(const lutgemm_weight *const *ws, const void *const *xs, 
  * group index is taken per weight and the offset is not dropped. */
 int lutgemm_dequantize(const lutgemm_weight *w, void *d_fW, int transposed, void *stream);
 
+/* Measurement aid without counterpart in the reference: for each of the `count` handles in turn,
+ * streams its packed tiles once with a kernel that only reads (same grid as that handle's launch
+ * plan, 16-byte loads, nothing written).  The time per launch is the device's pure-read time for
+ * the bytes a matvec has to fetch, the ceiling the benchmark quotes next to the matvec.
+ * Asynchronous on `stream`. */
+int lutgemm_read_probe(const lutgemm_weight *const *ws, int count, void *stream);
+
 /* Copy the packed planes back into the host input layout (exact inverse of the re-tiling):
  * bW [k/32][q][n] uint32, alpha [num_groups][q][n] and q_bias [num_groups][n] as binary16
  * bit patterns; any output pointer may be NULL to skip it.  Synchronous. */

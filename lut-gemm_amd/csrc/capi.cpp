@@ -536,6 +536,23 @@ int lutgemm_dequantize(const lutgemm_weight *w, void *d_fW, int transposed, void
     return LUTGEMM_OK;
 }
 
+int lutgemm_read_probe(const lutgemm_weight *const *ws, int count, void *stream)
+{
+    if (!ws) return fail(LUTGEMM_ERR_NULL_POINTER, "null argument to read_probe");
+    if (count < 0) return fail(LUTGEMM_ERR_BAD_SHAPE, "count=%d is negative", count);
+    for (int i = 0; i < count; i++) {
+        const lutgemm_weight *w = ws[i];
+        if (!w) return fail(LUTGEMM_ERR_NULL_POINTER, "null handle in read_probe");
+        if (int st_dev = check_device(w)) return st_dev;
+        const Shape &s = w->shape;
+        hipError_t e = lutgemm_kernels::launch_read_probe(w->d_signs, sign_bytes(s), w->d_scales, scale_bytes(s),
+                                                          w->plan.ntiles * w->plan.k_splits, w->plan.waves * kLanes,
+                                                          static_cast<hipStream_t>(stream));
+        if (e != hipSuccess) return hip_fail(e, "launch read_probe_kernel");
+    }
+    return LUTGEMM_OK;
+}
+
 int lutgemm_weight_unpack(const lutgemm_weight *w, uint32_t *bW, uint16_t *alpha, uint16_t *q_bias)
 {
     if (!w) return fail(LUTGEMM_ERR_NULL_POINTER, "null argument to weight_unpack");

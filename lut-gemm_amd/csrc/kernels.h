@@ -44,5 +44,9 @@ hipError_t launch_gather_columns(const void *cols, void *rows, int k, int m, hip
 
 hipError_t launch_dequantize(const DequantArgs &a, hipStream_t stream);
 
+// pure read of two byte ranges (multiples of 16 bytes), nothing written
+hipError_t launch_read_probe(const void *a, size_t bytes_a, const void *b, size_t bytes_b, int workgroups,
+                             int threads, hipStream_t stream);
+
 }  // namespace lutgemm_kernels
 #endif

@@ -749,6 +749,36 @@ __global__ __launch_bounds__(256) void dequantize_kernel(DequantArgs a)
     }
 }
 
+// Reads two byte ranges once with 16-byte non-temporal loads and does nothing else (the xor of
+// the data only feeds a store that never happens): the time of this kernel over a weight's tiles
+// is the device's pure-read time for the bytes the matvec has to stream.
+__device__ __forceinline__ unsigned read_range(const u32x4 *p, size_t n, size_t tid, size_t stride)
+{
+    constexpr int kInFlight = 6;  // loads per thread before the first use
+    unsigned acc = 0;
+    size_t i = tid;
+    for (; i + (kInFlight - 1) * stride < n; i += kInFlight * stride) {
+        u32x4 v[kInFlight];
+#pragma unroll
+        for (int u = 0; u < kInFlight; u++) v[u] = __builtin_nontemporal_load(p + i + u * stride);
+#pragma unroll
+        for (int u = 0; u < kInFlight; u++) acc ^= v[u].x ^ v[u].y ^ v[u].z ^ v[u].w;
+    }
+    for (; i < n; i += stride) {
+        const u32x4 v = __builtin_nontemporal_load(p + i);
+        acc ^= v.x ^ v.y ^ v.z ^ v.w;
+    }
+    return acc;
+}
+
+__global__ __launch_bounds__(768) void read_probe_kernel(const u32x4 *a, size_t na, const u32x4 *b, size_t nb,
+                                                         unsigned *never_written)
+{
+    const size_t tid = (size_t)blockIdx.x * blockDim.x + threadIdx.x, stride = (size_t)gridDim.x * blockDim.x;
+    const unsigned acc = read_range(a, na, tid, stride) ^ read_range(b, nb, tid, stride);
+    if (na + nb == 0 && acc == 0x12345678u) never_written[0] = acc;
+}
+
 // x [k][m] (m vectors stored as columns) -> rows [m][k], so that the matvec kernel can read
 // each vector with 16-byte loads.
 __global__ __launch_bounds__(256) void gather_columns_kernel(const uint16_t *cols, uint16_t *rows, int k, int m)
@@ -842,6 +872,15 @@ hipError_t launch_gather_columns(const void *cols, void *rows, int k, int m, hip
     const int threads = 256;
     hipLaunchKernelGGL(gather_columns_kernel, dim3((unsigned)((total + threads - 1) / threads)), dim3(threads),
                        0, stream, static_cast<const uint16_t *>(cols), static_cast<uint16_t *>(rows), k, m);
+    return hipGetLastError();
+}
+
+hipError_t launch_read_probe(const void *a, size_t bytes_a, const void *b, size_t bytes_b, int workgroups,
+                             int threads, hipStream_t stream)
+{
+    hipLaunchKernelGGL(read_probe_kernel, dim3(workgroups), dim3(threads), 0, stream,
+                       static_cast<const u32x4 *>(a), bytes_a / 16, static_cast<const u32x4 *>(b), bytes_b / 16,
+                       static_cast<unsigned *>(nullptr));
     return hipGetLastError();
 }
 

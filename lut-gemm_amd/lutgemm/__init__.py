@@ -30,7 +30,7 @@ EXPORTED = [
     "lutgemm_weight_plan", "lutgemm_weight_set_plan", "lutgemm_weight_autotune", "lutgemm_weight_device_ptrs", "lutgemm_packed_sizes",
     "lutgemm_pack_host", "lutgemm_unpack_host", "lutgemm_float_to_half", "lutgemm_last_error",
     "lutgemm_status_string", "lutgemm_version", "lutgemm_pack_file", "lutgemm_unpack_file", "lutgemm_weight_save",
-    "lutgemm_weight_load", "lutgemm_weight_clone",
+    "lutgemm_weight_load", "lutgemm_weight_clone", "lutgemm_read_probe",
 ]
 
 
@@ -87,6 +87,7 @@ def load():
     L.lutgemm_weight_save.argtypes = [vp, ctypes.c_char_p]
     L.lutgemm_weight_load.argtypes = [ctypes.c_char_p, pp]
     L.lutgemm_weight_clone.argtypes = [vp, pp]
+    L.lutgemm_read_probe.argtypes = [vp, i, vp]
     L.lutgemm_weight_set_plan.argtypes = [vp, i, i]
     L.lutgemm_weight_autotune.argtypes = [vp, vp]
     L.lutgemm_weight_device_ptrs.argtypes = [vp, pp, pp, pp]
@@ -306,6 +307,12 @@ class MatvecSequence:
 
     def launch(self, stream=0):
         _check(load().lutgemm_matvec_many(self._ws, self._xs, self._ys, self._ms, self.count, stream or None))
+
+
+def read_probe(weights, stream=0):
+    """Pure read of the packed tiles of each weight in turn (measurement aid), one C call."""
+    arr = (ctypes.c_void_p * len(weights))(*[w._h for w in weights])
+    _check(load().lutgemm_read_probe(arr, len(weights), stream or None))
 
 
 def version():

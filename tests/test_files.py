@@ -124,6 +124,9 @@ def test_file_entry_points_check_their_arguments(lutgemm, tmp_path):
     assert L.lutgemm_weight_clone(None, ctypes.byref(h)) == lutgemm.ERR_NULL_POINTER
     assert L.lutgemm_pack_file(None, None, None, 512, 8, 1, 1, b"/tmp/x.lutw") == lutgemm.ERR_NULL_POINTER
     assert L.lutgemm_unpack_file(None, None, None, None, None) == lutgemm.ERR_NULL_POINTER
+    assert L.lutgemm_read_probe(None, 1, None) == lutgemm.ERR_NULL_POINTER
+    assert L.lutgemm_read_probe((ctypes.c_void_p * 1)(None), 1, None) == lutgemm.ERR_NULL_POINTER
+    assert L.lutgemm_read_probe((ctypes.c_void_p * 1)(None), 0, None) == lutgemm.OK
     assert L.lutgemm_status_string(lutgemm.ERR_IO) == b"file input/output failed"
     assert h.value is None
     if not torch.cuda.is_available():
