@@ -182,7 +182,7 @@ def base_line(args, metric, value, us, workload, extra_config=None):
         "us_per_matvec": us, "pct_hbm_peak": 100.0 * value / HBM_PEAK_GBS,
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": None,
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-        "dtype": "fp16 in/out, fp32 accumulate",
+        "dtype": "fp16", "dtype_detail": "fp16 activations, scales and outputs; fp32 tables and accumulation",
         "data": "synthetic (seeded; Bernoulli signs, |N(0,0.02)| scales, N(0,1) fp16 activations)",
         "config": cfg,
     }
