@@ -1,0 +1,240 @@
+// gfx950 kernels that expand a packed BCQ weight to dense fp16.
+#include <hip/hip_fp16.h>
+#include <hip/hip_runtime.h>
+
+#include "device_util.h"
+#include "kernels.h"
+#include "layout.h"
+
+namespace lutgemm_kernels {
+using namespace lutgemm_layout;
+
+namespace {
+
+// ------------------------------------------------------------------------------------------
+// Dense fp16 weight from the packed tiles: W[k][n] or W[n][k], offset included.
+// One wavefront per tile (32 outputs x 512 k), lane L on chunk L as in the matvec: 2q coalesced
+// 16-byte sign loads and one scale record per lane, scales fetched across lanes with DPP, then
+// per weight the fp32 sum  offset +- alpha_0 +- alpha_1 ...  in plane order (the order of
+// lutGEMM::dequantize_cpu, lutGEMM/src/nQWeight_fp16.cu:38-59, so offset-free results are
+// bit-identical to it), one rounding to fp16, 16-byte stores: 8 consecutive k of one output
+// (a wavefront writes 1 KiB runs of a row of W[n][k]).  A workgroup is four wavefronts on four
+// neighbouring batches of the same k-block.  Used for W[n][k].
+// ------------------------------------------------------------------------------------------
+template <int GSUB, int LANE_IN_SUB>
+__device__ __forceinline__ float scale_from_holder(float v)
+{
+    const unsigned u = __builtin_bit_cast(unsigned, v);
+    if constexpr (GSUB == 1) {
+        return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0u, u, 0x150 + LANE_IN_SUB, 0xf, 0xf, false));
+    } else if constexpr (GSUB == 2) {
+        const unsigned lo = __builtin_amdgcn_update_dpp(0u, u, 0x150 + LANE_IN_SUB, 0xf, 0x3, false);
+        return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(lo, u, 0x150 + 8 + LANE_IN_SUB, 0xf, 0xc, false));
+    } else {
+        return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0u, u, LANE_IN_SUB * 0x55, 0xf, 0xf, false));
+    }
+}
+
+template <int Q, bool OFF, int GSUB>
+__global__ __launch_bounds__(256) void dequantize_kernel(DequantArgs a)
+{
+    constexpr int QO = Q + (OFF ? 1 : 0);
+    constexpr int SUBL = 16 / GSUB;
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int nbatches = (a.n + kBatch - 1) / kBatch;
+    // neighbouring workgroups write neighbouring memory: consecutive k-blocks of the same rows
+    const int ts = (int)(blockIdx.x % a.ts);
+    const int bg = (int)(blockIdx.x / a.ts);
+    const int nb = bg * 4 + wave;
+    if (nb >= nbatches) return;
+    const size_t tile = (size_t)nb * a.ts + ts;
+
+    const u32x4 *sp = reinterpret_cast<const u32x4 *>(a.signs) + tile * (size_t)(2 * Q * kLanes) + lane;
+    const uint32_t *cp = reinterpret_cast<const uint32_t *>(a.scales) + (tile * kLanes + lane) * (size_t)(GSUB * QO);
+    u32x4 sg[2 * Q];
+#pragma unroll
+    for (int u = 0; u < 2 * Q; u++) sg[u] = __builtin_nontemporal_load(sp + u * kLanes);
+    float sc[2 * GSUB * QO];  // [slot][plane or offset]
+#pragma unroll
+    for (int d = 0; d < GSUB * QO; d++) {
+        const uint32_t rec = __builtin_nontemporal_load(cp + d);
+        const __half2 h2 = *reinterpret_cast<const __half2 *>(&rec);
+        sc[2 * d] = __low2float(h2);
+        sc[2 * d + 1] = __high2float(h2);
+    }
+
+    const int kbase = ts * kBlockK + lane * kChunk;
+    const bool k_ok = kbase < a.k;  // k is a multiple of 32: a chunk is wholly inside or outside
+    __half *dst = reinterpret_cast<__half *>(a.out);
+
+    for (int h = 0; h < 2; h++) {  // the two halves of the batch: sign units (b, h), scale slots of that half
+        u32x4 sgh[Q];
+#pragma unroll
+        for (int b = 0; b < Q; b++) {
+            sgh[b].x = h ? sg[2 * b + 1].x : sg[2 * b].x;
+            sgh[b].y = h ? sg[2 * b + 1].y : sg[2 * b].y;
+            sgh[b].z = h ? sg[2 * b + 1].z : sg[2 * b].z;
+            sgh[b].w = h ? sg[2 * b + 1].w : sg[2 * b].w;
+        }
+        float sch[GSUB * QO];  // the GSUB slots of this half
+#pragma unroll
+        for (int d = 0; d < GSUB * QO; d++) sch[d] = h ? sc[GSUB * QO + d] : sc[d];
+        static_for<2>([&](auto P) {
+            constexpr int p0 = P * 8;  // outputs h*16 + p0 .. +7: bytes p0 .. p0+7 of the sign vectors
+            float w[8][8];             // [output][k]
+            static_for<8>([&](auto OI) {
+                constexpr int oi = OI;
+                constexpr int ih = p0 + oi;  // output within the half
+                float s[QO];
+#pragma unroll
+                for (int bo = 0; bo < QO; bo++) s[bo] = scale_from_holder<GSUB, ih % SUBL>(sch[(ih / SUBL) * QO + bo]);
+                uint32_t byte[Q];
+#pragma unroll
+                for (int b = 0; b < Q; b++) {
+                    const uint32_t word = ih / 4 == 0 ? sgh[b].x : ih / 4 == 1 ? sgh[b].y : ih / 4 == 2 ? sgh[b].z : sgh[b].w;
+                    byte[b] = (word >> ((ih % 4) * 8)) & 0xffu;
+                }
+#pragma unroll
+                for (int t = 0; t < 8; t++) {
+                    float v = OFF ? s[Q] : 0.f;
+#pragma unroll
+                    for (int b = 0; b < Q; b++) v += ((byte[b] >> t) & 1u) ? s[b] : -s[b];
+                    w[oi][t] = v;
+                }
+            });
+            const int col0 = nb * kBatch + h * 16 + p0;  // first of the 8 outputs
+#pragma unroll
+            for (int oi = 0; oi < 8; oi++) {
+                if (k_ok && col0 + oi < a.n) {
+                    __half2 hh[4];
+#pragma unroll
+                    for (int t2 = 0; t2 < 4; t2++) hh[t2] = __floats2half2_rn(w[oi][2 * t2], w[oi][2 * t2 + 1]);
+                    u32x4 v;
+                    v.x = *reinterpret_cast<uint32_t *>(&hh[0]);
+                    v.y = *reinterpret_cast<uint32_t *>(&hh[1]);
+                    v.z = *reinterpret_cast<uint32_t *>(&hh[2]);
+                    v.w = *reinterpret_cast<uint32_t *>(&hh[3]);
+                    *reinterpret_cast<u32x4 *>(dst + (size_t)(col0 + oi) * a.k + kbase) = v;
+                }
+            }
+        });
+    }
+}
+
+// W[k][n] (and either orientation by its `transposed` branch): one thread per (chunk, output),
+// consecutive threads on consecutive outputs, 2-byte stores that a wavefront coalesces into
+// 128-byte runs.  Same arithmetic.  Writing W[k][n] from the tile kernel's lanes would scatter
+// 16-byte pieces over 64 rows per store instruction, which measured slower than this.
+__global__ __launch_bounds__(256) void dequantize_generic_kernel(DequantArgs a)
+{
+    const int qo = a.q + a.has_offset;
+    const int subl = 16 / a.gsub;
+    const int lh = 2 * a.gsub * qo;
+    const size_t chunks = (size_t)a.k / kChunk;
+    const size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx >= chunks * (size_t)a.n) return;
+    int out, c;
+    if (a.transposed) {  // consecutive threads -> consecutive chunks of one output row
+        c = (int)(idx % chunks);
+        out = (int)(idx / chunks);
+    } else {             // consecutive threads -> consecutive outputs of one chunk
+        out = (int)(idx % (size_t)a.n);
+        c = (int)(idx / (size_t)a.n);
+    }
+    const int nb = out / kBatch, i = out % kBatch, h = i / 16, p = i % 16;
+    const int ts = c / kLanes, lane = c % kLanes;
+    const size_t tile = (size_t)nb * a.ts + ts;
+    const int r = lane / 16, j = lane % 16, sub = j / subl;
+    // lane of the same sub-row that holds this output's scales, and the slot inside it
+    const int holder = r * 16 + sub * subl + (i % subl);
+    const int slot = i / subl;
+    const __half *sc =
+        reinterpret_cast<const __half *>(a.scales) + (tile * kLanes + holder) * (size_t)lh + slot * qo;
+    float w[8];
+    const float off = a.has_offset ? __half2float(sc[a.q]) : 0.f;
+#pragma unroll
+    for (int t = 0; t < 8; t++) w[t] = off;
+    for (int b = 0; b < a.q; b++) {
+        const uint8_t byte = a.signs[(tile * (size_t)(2 * a.q) + 2 * b + h) * kUnitBytes + lane * 16 + p];
+        const float al = __half2float(sc[b]);
+#pragma unroll
+        for (int t = 0; t < 8; t++) w[t] += ((byte >> t) & 1) ? al : -al;
+    }
+    __half *dst = reinterpret_cast<__half *>(a.out);
+    if (a.transposed) {
+        __half hv[8];
+#pragma unroll
+        for (int t = 0; t < 8; t++) hv[t] = __float2half_rn(w[t]);
+        *reinterpret_cast<uint4 *>(dst + (size_t)out * a.k + (size_t)c * kChunk) =
+            *reinterpret_cast<const uint4 *>(hv);
+    } else {
+#pragma unroll
+        for (int t = 0; t < 8; t++) dst[((size_t)c * kChunk + t) * a.n + out] = __float2half_rn(w[t]);
+    }
+}
+
+}  // namespace
+
+namespace {
+template <int Q, bool OFF>
+hipError_t launch_dequantize_gsub(const DequantArgs &a, unsigned blocks, hipStream_t stream)
+{
+    switch (a.gsub) {
+        case 1: hipLaunchKernelGGL((dequantize_kernel<Q, OFF, 1>), dim3(blocks), dim3(256), 0, stream, a); break;
+        case 2: hipLaunchKernelGGL((dequantize_kernel<Q, OFF, 2>), dim3(blocks), dim3(256), 0, stream, a); break;
+        default: hipLaunchKernelGGL((dequantize_kernel<Q, OFF, 4>), dim3(blocks), dim3(256), 0, stream, a); break;
+    }
+    return hipGetLastError();
+}
+template <int Q>
+hipError_t launch_dequantize_q(const DequantArgs &a, unsigned blocks, hipStream_t stream)
+{
+    return a.has_offset ? launch_dequantize_gsub<Q, true>(a, blocks, stream)
+                        : launch_dequantize_gsub<Q, false>(a, blocks, stream);
+}
+}  // namespace
+
+hipError_t launch_dequantize(const DequantArgs &a, hipStream_t stream)
+{
+    if (!a.transposed) {
+        const size_t total = (size_t)(a.k / kChunk) * (size_t)a.n;
+        const size_t blocks = (total + 255) / 256;
+        if (blocks > 0x7fffffffu) return hipErrorInvalidValue;
+        hipLaunchKernelGGL(dequantize_generic_kernel, dim3((unsigned)blocks), dim3(256), 0, stream, a);
+        return hipGetLastError();
+    }
+    const size_t nbatches = ((size_t)a.n + kBatch - 1) / kBatch;
+    const size_t blocks = ((nbatches + 3) / 4) * (size_t)a.ts;
+    if (blocks > 0x7fffffffu) return hipErrorInvalidValue;
+    const unsigned nblk = (unsigned)blocks;
+    switch (a.q) {
+#if !defined(LUTGEMM_DEV_ONLY_Q) || LUTGEMM_DEV_ONLY_Q == 1
+        case 1: return launch_dequantize_q<1>(a, nblk, stream);
+#endif
+#if !defined(LUTGEMM_DEV_ONLY_Q) || LUTGEMM_DEV_ONLY_Q == 2
+        case 2: return launch_dequantize_q<2>(a, nblk, stream);
+#endif
+#if !defined(LUTGEMM_DEV_ONLY_Q) || LUTGEMM_DEV_ONLY_Q == 3
+        case 3: return launch_dequantize_q<3>(a, nblk, stream);
+#endif
+#if !defined(LUTGEMM_DEV_ONLY_Q) || LUTGEMM_DEV_ONLY_Q == 4
+        case 4: return launch_dequantize_q<4>(a, nblk, stream);
+#endif
+#if !defined(LUTGEMM_DEV_ONLY_Q) || LUTGEMM_DEV_ONLY_Q == 5
+        case 5: return launch_dequantize_q<5>(a, nblk, stream);
+#endif
+#if !defined(LUTGEMM_DEV_ONLY_Q) || LUTGEMM_DEV_ONLY_Q == 6
+        case 6: return launch_dequantize_q<6>(a, nblk, stream);
+#endif
+#if !defined(LUTGEMM_DEV_ONLY_Q) || LUTGEMM_DEV_ONLY_Q == 7
+        case 7: return launch_dequantize_q<7>(a, nblk, stream);
+#endif
+#if !defined(LUTGEMM_DEV_ONLY_Q) || LUTGEMM_DEV_ONLY_Q == 8
+        case 8: return launch_dequantize_q<8>(a, nblk, stream);
+#endif
+        default: return hipErrorInvalidValue;
+    }
+}
+
+}  // namespace lutgemm_kernels

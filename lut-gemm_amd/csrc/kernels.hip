@@ -27,6 +27,7 @@
 #include <type_traits>
 #include <utility>
 
+#include "device_util.h"
 #include "kernels.h"
 #include "layout.h"
 
@@ -36,20 +37,6 @@ using namespace lutgemm_layout;
 namespace {
 
 constexpr int kTableFloats = 256 * kLanes;  // one table set: 64 KiB
-
-typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
-
-// compile-time loop: body(std::integral_constant<int, I>) for I in [0, N)
-template <typename F, int... Is>
-__device__ __forceinline__ void static_for_impl(F &&body, std::integer_sequence<int, Is...>)
-{
-    (body(std::integral_constant<int, Is>{}), ...);
-}
-template <int N, typename F>
-__device__ __forceinline__ void static_for(F &&body)
-{
-    static_for_impl(body, std::make_integer_sequence<int, N>{});
-}
 
 // ------------------------------------------------------------------------------------------
 // Eight table lookups with their scaled accumulation, written in GCN assembly so that a lookup
@@ -697,58 +684,6 @@ __global__ __launch_bounds__(768) void lut_matvec2_kernel(MatvecArgs a)
     finish_output(total1, active && a.rows > 1, out, lane, y + a.y_row_stride, a.accum + a.accum_row_stride, a);
 }
 
-// ------------------------------------------------------------------------------------------
-// Dense fp16 weight from the packed tiles: W[k][n] or W[n][k], offset included.
-// One thread per (chunk, output): reads its q sign bytes and scales, writes 8 weights.
-// ------------------------------------------------------------------------------------------
-__global__ __launch_bounds__(256) void dequantize_kernel(DequantArgs a)
-{
-    const int qo = a.q + a.has_offset;
-    const int subl = 16 / a.gsub;
-    const int lh = 2 * a.gsub * qo;
-    const size_t chunks = (size_t)a.k / kChunk;
-    const size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
-    if (idx >= chunks * (size_t)a.n) return;
-    int out, c;
-    if (a.transposed) {  // consecutive threads -> consecutive chunks of one output row
-        c = (int)(idx % chunks);
-        out = (int)(idx / chunks);
-    } else {             // consecutive threads -> consecutive outputs of one chunk
-        out = (int)(idx % (size_t)a.n);
-        c = (int)(idx / (size_t)a.n);
-    }
-    const int nb = out / kBatch, i = out % kBatch, h = i / 16, p = i % 16;
-    const int ts = c / kLanes, lane = c % kLanes;
-    const size_t tile = (size_t)nb * a.ts + ts;
-    const int r = lane / 16, j = lane % 16, sub = j / subl;
-    // lane of the same sub-row that holds this output's scales, and the slot inside it
-    const int holder = r * 16 + sub * subl + (i % subl);
-    const int slot = i / subl;
-    const __half *sc =
-        reinterpret_cast<const __half *>(a.scales) + (tile * kLanes + holder) * (size_t)lh + slot * qo;
-    float w[8];
-    const float off = a.has_offset ? __half2float(sc[a.q]) : 0.f;
-#pragma unroll
-    for (int t = 0; t < 8; t++) w[t] = off;
-    for (int b = 0; b < a.q; b++) {
-        const uint8_t byte = a.signs[(tile * (size_t)(2 * a.q) + 2 * b + h) * kUnitBytes + lane * 16 + p];
-        const float al = __half2float(sc[b]);
-#pragma unroll
-        for (int t = 0; t < 8; t++) w[t] += ((byte >> t) & 1) ? al : -al;
-    }
-    __half *dst = reinterpret_cast<__half *>(a.out);
-    if (a.transposed) {
-        __half hv[8];
-#pragma unroll
-        for (int t = 0; t < 8; t++) hv[t] = __float2half_rn(w[t]);
-        *reinterpret_cast<uint4 *>(dst + (size_t)out * a.k + (size_t)c * kChunk) =
-            *reinterpret_cast<const uint4 *>(hv);
-    } else {
-#pragma unroll
-        for (int t = 0; t < 8; t++) dst[((size_t)c * kChunk + t) * a.n + out] = __float2half_rn(w[t]);
-    }
-}
-
 // Reads two byte ranges once with 16-byte non-temporal loads and does nothing else (the xor of
 // the data only feeds a store that never happens): the time of this kernel over a weight's tiles
 // is the device's pure-read time for the bytes the matvec has to stream.
@@ -881,16 +816,6 @@ hipError_t launch_read_probe(const void *a, size_t bytes_a, const void *b, size_
     hipLaunchKernelGGL(read_probe_kernel, dim3(workgroups), dim3(threads), 0, stream,
                        static_cast<const u32x4 *>(a), bytes_a / 16, static_cast<const u32x4 *>(b), bytes_b / 16,
                        static_cast<unsigned *>(nullptr));
-    return hipGetLastError();
-}
-
-hipError_t launch_dequantize(const DequantArgs &a, hipStream_t stream)
-{
-    const size_t total = (size_t)(a.k / kChunk) * (size_t)a.n;
-    const int threads = 256;
-    const size_t blocks = (total + threads - 1) / threads;
-    if (blocks > 0x7fffffffu) return hipErrorInvalidValue;
-    hipLaunchKernelGGL(dequantize_kernel, dim3((unsigned)blocks), dim3(threads), 0, stream, a);
     return hipGetLastError();
 }
 

@@ -101,17 +101,18 @@ class LutLinear(torch.nn.Module):
         return cls(c, bias=b, **kw)
 
     def dense_weight(self):
-        """Dequantised fp16 W [k][n] on the device (built once, kept for large batches)."""
+        """Dequantised fp16 weight on the device as W^T [n][k] (built once, kept for large
+        batches): the orientation the dequantise kernel writes in 1 KiB runs."""
         if self._dense is None:
-            W = torch.empty((self.in_features, self.out_features), dtype=torch.float16, device="cuda")
-            self.weight.dequantize(W.data_ptr(), False, torch.cuda.current_stream().cuda_stream)
-            self._dense = W
+            Wt = torch.empty((self.out_features, self.in_features), dtype=torch.float16, device="cuda")
+            self.weight.dequantize(Wt.data_ptr(), True, torch.cuda.current_stream().cuda_stream)
+            self._dense = Wt
         return self._dense
 
     def forward(self, x):
         rows = x.numel() // x.shape[-1]
         if rows > self.dense_threshold:
-            y = x.to(torch.float16) @ self.dense_weight()
+            y = torch.nn.functional.linear(x.to(torch.float16), self.dense_weight())
         else:
             y = torch.ops.lutgemm.matvec(x, self.handle)
         return y if self.bias is None else y + self.bias

@@ -44,13 +44,13 @@ def test_large_batches_take_the_dense_route(lutgemm, oracle, device):
     layer = torch_ops.LutLinear(c, dense_threshold=8)
     x = torch.randn(40, 1024, generator=gen).to(torch.float16)
     y_dense = layer(x.to(device))                       # 40 rows > threshold: dequantise + GEMM
-    assert layer._dense is not None and layer._dense.shape == (1024, 320)
+    assert layer._dense is not None and layer._dense.shape == (320, 1024)   # W^T [n][k]
     y_lut = torch.ops.lutgemm.matvec(x.to(device), layer.handle)
     # the dense weight is the oracle's dense weight rounded to fp16
     a16 = c["alpha"].astype(np.float16)
     z16 = c["q_bias"].astype(np.float16)
     dense = oracle.dense_weight_f64(c["bW"], a16, z16)
-    assert np.array_equal(layer._dense.cpu().numpy(), dense.astype(np.float16))
+    assert np.array_equal(layer._dense.cpu().numpy(), dense.T.astype(np.float16))
     truth = x.double().numpy() @ dense
     assert np.abs(y_lut.cpu().double().numpy() - truth).max() <= 1e-2
     assert np.abs(y_dense.cpu().double().numpy() - truth).max() <= 3e-2   # fp16 weight + library GEMM
