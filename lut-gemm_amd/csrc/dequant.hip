@@ -19,7 +19,7 @@ namespace {
 // lutGEMM::dequantize_cpu, lutGEMM/src/nQWeight_fp16.cu:38-59, so offset-free results are
 // bit-identical to it), one rounding to fp16, 16-byte stores: 8 consecutive k of one output
 // (a wavefront writes 1 KiB runs of a row of W[n][k]).  A workgroup is four wavefronts on four
-// neighbouring batches of the same k-block.  Used for W[n][k].
+// neighbouring batches of the same k-block.  Writes W[n][k].
 // ------------------------------------------------------------------------------------------
 template <int GSUB, int LANE_IN_SUB>
 __device__ __forceinline__ float scale_from_holder(float v)
@@ -97,7 +97,8 @@ __global__ __launch_bounds__(256) void dequantize_kernel(DequantArgs a)
                 }
 #pragma unroll
                 for (int t = 0; t < 8; t++) {
-                    float v = OFF ? s[Q] : 0.f;
+                    float v = 0.f;
+                    if constexpr (OFF) v = s[QO - 1];
 #pragma unroll
                     for (int b = 0; b < Q; b++) v += ((byte[b] >> t) & 1u) ? s[b] : -s[b];
                     w[oi][t] = v;
@@ -122,26 +123,80 @@ __global__ __launch_bounds__(256) void dequantize_kernel(DequantArgs a)
     }
 }
 
-// W[k][n] (and either orientation by its `transposed` branch): one thread per (chunk, output),
-// consecutive threads on consecutive outputs, 2-byte stores that a wavefront coalesces into
-// 128-byte runs.  Same arithmetic.  Writing W[k][n] from the tile kernel's lanes would scatter
-// 16-byte pieces over 64 rows per store instruction, which measured slower than this.
+// W[k][n], n a multiple of 8: one thread per (chunk, 8 consecutive outputs).  The 64 lanes of a
+// wavefront take 64 consecutive output groups of one chunk, so each of its eight 16-byte stores
+// (one per k of the chunk) writes a 1 KiB run of one row; the four wavefronts of a workgroup take
+// four consecutive chunks, which together use every byte of the 64-byte sign sectors they touch.
+// Sign bytes of 8 outputs are one 8-byte load per plane; scales are 2-byte loads shared through
+// the cache by the lanes of the same k-group.  Same arithmetic and order as the tile kernel.
+__global__ __launch_bounds__(256) void dequantize_rows_kernel(DequantArgs a)
+{
+    const int qo = a.q + a.has_offset;
+    const int subl = 16 / a.gsub;
+    const int lh = 2 * a.gsub * qo;
+    const int groups = a.n / 8;
+    const int group_blocks = (groups + 63) / 64;
+    const int og = (int)(blockIdx.x % group_blocks) * 64 + (int)(threadIdx.x & 63);
+    const int c = (int)(blockIdx.x / group_blocks) * 4 + (int)(threadIdx.x >> 6);
+    if (og >= groups || c >= a.k / kChunk) return;
+    const int out0 = og * 8;
+    const int nb = out0 / kBatch, i0 = out0 % kBatch, h = i0 / 16, p0 = i0 % 16;
+    const int ts = c / kLanes, lane = c % kLanes;
+    const size_t tile = (size_t)nb * a.ts + ts;
+    const int r = lane / 16, sub = (lane % 16) / subl;
+    const __half *sc_tile = reinterpret_cast<const __half *>(a.scales) + tile * kLanes * (size_t)lh;
+    // scale record of output i0 + oi: the lane of this k-group that holds it, and the slot in it
+    const __half *sc[8];
+#pragma unroll
+    for (int oi = 0; oi < 8; oi++) {
+        const int i = i0 + oi;
+        sc[oi] = sc_tile + (size_t)(r * 16 + sub * subl + (i % subl)) * lh + (i / subl) * qo;
+    }
+    float w[8][8];  // [output][k]
+#pragma unroll
+    for (int oi = 0; oi < 8; oi++) {
+        const float off = a.has_offset ? __half2float(sc[oi][a.q]) : 0.f;
+#pragma unroll
+        for (int t = 0; t < 8; t++) w[oi][t] = off;
+    }
+    const uint8_t *sg = a.signs + (tile * (size_t)(2 * a.q) + h) * kUnitBytes + lane * 16 + p0;
+    for (int b = 0; b < a.q; b++) {
+        const uint64_t bytes = *reinterpret_cast<const uint64_t *>(sg + (size_t)(2 * b) * kUnitBytes);
+#pragma unroll
+        for (int oi = 0; oi < 8; oi++) {
+            const float al = __half2float(sc[oi][b]);
+            const uint32_t byte = (uint32_t)(bytes >> (8 * oi)) & 0xffu;
+#pragma unroll
+            for (int t = 0; t < 8; t++) w[oi][t] += ((byte >> t) & 1u) ? al : -al;
+        }
+    }
+    __half *dst = reinterpret_cast<__half *>(a.out) + (size_t)c * kChunk * a.n + out0;
+#pragma unroll
+    for (int t = 0; t < 8; t++) {
+        __half2 hh[4];
+#pragma unroll
+        for (int o2 = 0; o2 < 4; o2++) hh[o2] = __floats2half2_rn(w[2 * o2][t], w[2 * o2 + 1][t]);
+        u32x4 v;
+        v.x = *reinterpret_cast<uint32_t *>(&hh[0]);
+        v.y = *reinterpret_cast<uint32_t *>(&hh[1]);
+        v.z = *reinterpret_cast<uint32_t *>(&hh[2]);
+        v.w = *reinterpret_cast<uint32_t *>(&hh[3]);
+        *reinterpret_cast<u32x4 *>(dst + (size_t)t * a.n) = v;
+    }
+}
+
+// W[k][n] for any n (rows of W are only 2-byte aligned when n is odd): one thread per (chunk,
+// output), consecutive threads on consecutive outputs, 2-byte stores that a wavefront coalesces
+// into 128-byte runs.  Same arithmetic.
 __global__ __launch_bounds__(256) void dequantize_generic_kernel(DequantArgs a)
 {
     const int qo = a.q + a.has_offset;
     const int subl = 16 / a.gsub;
     const int lh = 2 * a.gsub * qo;
-    const size_t chunks = (size_t)a.k / kChunk;
     const size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
-    if (idx >= chunks * (size_t)a.n) return;
-    int out, c;
-    if (a.transposed) {  // consecutive threads -> consecutive chunks of one output row
-        c = (int)(idx % chunks);
-        out = (int)(idx / chunks);
-    } else {             // consecutive threads -> consecutive outputs of one chunk
-        out = (int)(idx % (size_t)a.n);
-        c = (int)(idx / (size_t)a.n);
-    }
+    if (idx >= (size_t)(a.k / kChunk) * (size_t)a.n) return;
+    const int out = (int)(idx % (size_t)a.n);
+    const int c = (int)(idx / (size_t)a.n);
     const int nb = out / kBatch, i = out % kBatch, h = i / 16, p = i % 16;
     const int ts = c / kLanes, lane = c % kLanes;
     const size_t tile = (size_t)nb * a.ts + ts;
@@ -162,16 +217,8 @@ __global__ __launch_bounds__(256) void dequantize_generic_kernel(DequantArgs a)
         for (int t = 0; t < 8; t++) w[t] += ((byte >> t) & 1) ? al : -al;
     }
     __half *dst = reinterpret_cast<__half *>(a.out);
-    if (a.transposed) {
-        __half hv[8];
 #pragma unroll
-        for (int t = 0; t < 8; t++) hv[t] = __float2half_rn(w[t]);
-        *reinterpret_cast<uint4 *>(dst + (size_t)out * a.k + (size_t)c * kChunk) =
-            *reinterpret_cast<const uint4 *>(hv);
-    } else {
-#pragma unroll
-        for (int t = 0; t < 8; t++) dst[((size_t)c * kChunk + t) * a.n + out] = __float2half_rn(w[t]);
-    }
+    for (int t = 0; t < 8; t++) dst[((size_t)c * kChunk + t) * a.n + out] = __float2half_rn(w[t]);
 }
 
 }  // namespace
@@ -197,6 +244,12 @@ hipError_t launch_dequantize_q(const DequantArgs &a, unsigned blocks, hipStream_
 
 hipError_t launch_dequantize(const DequantArgs &a, hipStream_t stream)
 {
+    if (!a.transposed && a.n % 8 == 0) {
+        const size_t blocks = (size_t)((a.n / 8 + 63) / 64) * (size_t)(a.k / kChunk / 4);
+        if (blocks > 0x7fffffffu) return hipErrorInvalidValue;
+        hipLaunchKernelGGL(dequantize_rows_kernel, dim3((unsigned)blocks), dim3(256), 0, stream, a);
+        return hipGetLastError();
+    }
     if (!a.transposed) {
         const size_t total = (size_t)(a.k / kChunk) * (size_t)a.n;
         const size_t blocks = (total + 255) / 256;

@@ -152,6 +152,232 @@ def test_bit_order_of_container_words():
     assert np.array_equal(c["bW"], want)
 
 
+def test_weight_factors_closed_form():
+    """examples/bcq.py:52-76 on four weights worked by hand."""
+    x = torch.tensor([[1.0, -2.0, 3.0, -4.0]])
+    assert Q._weight_factors(x.clone(), 0.0, 1.0, 0.0) is None
+    # clipping 0.5: threshold = sorted |w| [int(4*0.5)] = 3; factor = |w|/3 saturated at 1
+    wf = Q._weight_factors(x.clone(), 0.0, 0.5, 0.0)
+    assert torch.allclose(wf, torch.tensor([[1 / 3, 2 / 3, 1.0, 1.0]]))
+    # exponent 2 on |w| / max|w|
+    wf = Q._weight_factors(x.clone(), 2.0, 1.0, 0.0)
+    assert torch.allclose(wf, torch.tensor([[1 / 16, 4 / 16, 9 / 16, 1.0]]))
+    # pruning 0.5: threshold = sorted |w| [2] = 3: |w| <= 3 gets factor 0 and is zeroed
+    xx = x.clone()
+    wf = Q._weight_factors(xx, 0.0, 1.0, 0.5)
+    assert torch.equal(wf, torch.tensor([[0.0, 0.0, 0.0, 1.0]]))
+    assert torch.equal(xx, torch.tensor([[0.0, 0.0, 0.0, -4.0]]))
+
+
+def test_weighted_greedy_and_least_squares():
+    gen = torch.Generator().manual_seed(2)
+    x = torch.randn(6, 32, generator=gen)
+    wf = torch.rand(6, 32, generator=gen) + 0.1
+    # one plane: the weighted least-squares scale for b = sign(w) is sum wf |w| / sum wf
+    B, A = Q._greedy(x, 1, wf)
+    assert torch.allclose(A[:, 0], (wf * x.abs()).sum(1) / wf.sum(1), rtol=1e-6)
+    # refinement: for the signs it is given, the new scales satisfy the weighted normal equations
+    # B^T diag(wf) (x - B a) = 0 (weights built from sorted positive scales, so |.| and the sort
+    # leave them alone), and an unweighted solve does not
+    pats = torch.where(torch.rand(6, 32, 3, generator=gen) > 0.5, 1.0, -1.0)
+    a_true = torch.tensor([0.9, 0.5, 0.2]).expand(6, 3)
+    xw = torch.einsum("rgq,rq->rg", pats, a_true) + 0.05 * torch.randn(6, 32, generator=gen)
+    _, A1 = Q._refine(xw, pats, a_true.clone(), wf, use_bst=True)
+    resid = xw - torch.einsum("rgq,rq->rg", pats, A1)
+    grad = torch.einsum("rgq,rg->rq", pats, wf * resid)
+    assert grad.abs().max() < 1e-3
+    _, A0 = Q._refine(xw, pats, a_true.clone(), None, use_bst=True)
+    resid0 = xw - torch.einsum("rgq,rq->rg", pats, A0)
+    assert torch.einsum("rgq,rg->rq", pats, wf * resid0).abs().max() > 1e-2
+    # a zero factor everywhere in a group gives scale 0, not NaN
+    wz = wf.clone()
+    wz[0] = 0.0
+    _, Az = Q._greedy(x, 2, wz)
+    assert torch.equal(Az[0], torch.zeros(2)) and torch.isfinite(Az).all()
+
+
+def test_quantize_options():
+    gen = torch.Generator().manual_seed(3)
+    w = torch.randn(48, 128, generator=gen)
+    base, Bb, Ab, kept = Q.quantize(w, 3, rounds=4, group_size=64)
+    assert kept.all() and Bb.shape == (48, 2, 64, 3) and Ab.shape == (48, 2, 3)
+    w3, B3, A3 = Q.bcq_quantize(w, 3, rounds=4, group_size=64)
+    assert torch.equal(w3, base) and torch.equal(B3, Bb) and torch.equal(A3, Ab)
+    # transpose: groups along the first dimension = the plain call on w.T
+    wt, Bt, At, _ = Q.quantize(w, 3, rounds=4, group_size=16, transpose=True)
+    w2, B2, A2, _ = Q.quantize(w.t().contiguous(), 3, rounds=4, group_size=16)
+    assert Bt.shape == (128, 3, 16, 3) and torch.equal(Bt, B2) and torch.equal(At, A2) and torch.equal(wt, w2.t())
+    # greedy sign assignment: plane 0 is the sign of the weight, plane i the sign of the residual
+    wg, Bg, Ag, _ = Q.quantize(w, 3, rounds=3, group_size=64, use_bst=False)
+    x = w.reshape(-1, 64)
+    Bg2, Ag2 = Bg.reshape(-1, 64, 3), Ag.reshape(-1, 3)
+    r = x.clone()
+    for i in range(3):
+        assert torch.equal(Bg2[:, :, i], torch.where(r >= 0, 1.0, -1.0))
+        r -= Bg2[:, :, i] * Ag2[:, i:i + 1]
+    # the nearest-level assignment is never worse than the greedy one for the same scales
+    assert (base - w).pow(2).sum() <= (wg - w).pow(2).sum() * 1.001
+    # pruning: that fraction of the smallest weights is dropped: code 0 in every plane, value 0
+    wp, Bp, Ap, keptp = Q.quantize(w, 3, rounds=3, group_size=64, pruning=0.25)
+    frac = 1.0 - keptp.float().mean().item()
+    assert abs(frac - 0.25) < 0.01
+    dropped = ~keptp.reshape(48, 2, 64)
+    assert (Bp[dropped] == 0).all() and (Bp[~dropped].abs() == 1).all()
+    assert (wp.reshape(48, 2, 64)[dropped] == 0).all()
+    assert w.abs().reshape(48, 2, 64)[dropped].max() <= w.abs().reshape(48, 2, 64)[~dropped].min()
+    with pytest.raises(ValueError, match="zeros"):
+        Q.to_container(Bp, Ap)
+    # importance weighting moves error away from the large weights
+    we, _, _, _ = Q.quantize(w, 2, rounds=6, group_size=64, exponent=2.0)
+    wu, _, _, _ = Q.quantize(w, 2, rounds=6, group_size=64)
+    big = w.abs() > w.abs().quantile(0.9)
+    assert (we - w)[big].pow(2).mean() < (wu - w)[big].pow(2).mean()
+
+
+def test_packer_known_answer_and_round_trip():
+    """examples/utils.py:164-183: entry i*N/8 + j of the flattened tensor is bit i of byte j."""
+    b = -torch.ones(2, 8)            # N = 16, two bytes
+    b[0, 0] = 1                      # flat 0  = 0*2 + 0 -> byte 0 bit 0
+    b[0, 3] = 1                      # flat 3  = 1*2 + 1 -> byte 1 bit 1
+    b[1, 6] = 1                      # flat 14 = 7*2 + 0 -> byte 0 bit 7
+    pb, shape = Q.PACKER.pack(b)
+    assert pb.dtype == torch.uint8 and pb.tolist() == [0x81, 0x02] and tuple(shape) == (2, 8)
+    assert torch.equal(Q.PACKER.unpack(pb, shape, torch.float32), b)
+    gen = torch.Generator().manual_seed(4)
+    r = torch.where(torch.rand(3, 4, 16, 2, generator=gen) > 0.5, 1.0, -1.0)
+    pr, sh = Q.PACKER.pack(r)
+    assert pr.numel() == r.numel() // 8 and torch.equal(Q.PACKER.unpack(pr, sh, torch.float32), r)
+
+
+@pytest.mark.parametrize("in_ch_wise", [False, True])
+def test_parameter_classes_follow_the_example_flow(in_ch_wise):
+    """The flow of the reference's examples (examples/rtn_parameter.py:98-112,
+    examples/bcq_parameter.py:70-81): RTN compress -> decompress, conversion to BCQ with and
+    without packing, BCQ decompress of the converted codes equals the RTN decompress."""
+    gen = torch.Generator().manual_seed(6)
+    w_org = torch.randn(64, 256, generator=gen)
+    w_rtn = Q.RTNParameter(w_org)
+    scale, zero, codes, shape = w_rtn.compress(in_ch_wise=in_ch_wise, qbits=4, group_size=32, perchannel=True, sym=False)
+    d0 = 256 if in_ch_wise else 64
+    assert tuple(shape) == (d0, (64 * 256 // d0) // 32, 32) and scale.shape == (d0, shape[1], 1)
+    w_rtn.decompress(scale, zero, codes, shape, in_ch_wise=in_ch_wise)
+    assert w_rtn.data.shape == (64, 256)
+    assert (w_rtn.data - w_org).abs().max() <= scale.max() * 0.5001
+    for packing in (False, True):
+        alpha, binary, bshape, offset = w_rtn.convert_bcq_format(scale, zero, codes, qbits=4, do_packing=packing,
+                                                                 in_ch_wise=in_ch_wise)
+        assert tuple(bshape) == tuple(shape) + (4,)
+        assert binary.dtype == (torch.uint8 if packing else torch.float32)
+        w_bcq = Q.BCQParameter(w_org)
+        w_bcq.decompress(alpha, binary, bshape, offset=offset, do_packing=packing, in_ch_wise=in_ch_wise)
+        assert torch.allclose(w_bcq.data, w_rtn.data, atol=1e-5)
+    w_bcq = Q.BCQParameter(w_org)
+    alpha, binary, bshape = w_bcq.compress(do_packing=True, in_ch_wise=in_ch_wise, qbits=3, rounds=4, group_size=32)
+    assert alpha.shape == (d0, shape[1], 3) and binary.numel() == 64 * 256 * 3 // 8
+    w_bcq.decompress(alpha, binary, bshape, do_packing=True, in_ch_wise=in_ch_wise)
+    assert w_bcq.data.shape == (64, 256) and (w_bcq.data - w_org).abs().mean() < 0.2
+
+
+def test_rtn_whole_tensor_range():
+    """perchannel=False: one (scale, zero) for the whole tensor (examples/utils.py:69-70)."""
+    gen = torch.Generator().manual_seed(7)
+    w = torch.randn(8, 64, generator=gen)
+    scale, zero, codes = Q.rtn_quantize(w, 4, group_size=32, perchannel=False)
+    assert scale.shape == (8, 2, 1) and (scale == scale.flatten()[0]).all() and (zero == zero.flatten()[0]).all()
+    assert torch.isclose(scale.flatten()[0], (w.max() - w.min()) / 15)
+    assert (Q.rtn_dequantize(scale, zero, codes) - w).abs().max() <= scale.flatten()[0] * 0.5001
+
+
+class _Block(torch.nn.Module):
+    def __init__(self, d, f, bias):
+        super().__init__()
+        self.q_proj = torch.nn.Linear(d, d, bias=bias)
+        self.fc1 = torch.nn.Linear(d, f, bias=bias)
+        self.fc2 = torch.nn.Linear(f, d, bias=bias)
+        self.gate = torch.nn.Linear(d, d)      # not one of the converted names
+        self.norm = torch.nn.LayerNorm(d)
+
+    def forward(self, x):
+        h = self.norm(x)
+        h = x + self.q_proj(h)
+        return h + self.fc2(torch.relu(self.fc1(h)))
+
+
+def test_quantize_model_finds_the_projection_layers():
+    torch.manual_seed(8)
+    model = torch.nn.Sequential(_Block(64, 128, True), _Block(64, 128, False))
+    found = Q.quantize_model(model, qbits=3, group_size=32, method="rtn", to_device=False)
+    assert sorted(found) == ["0.fc1", "0.fc2", "0.q_proj", "1.fc1", "1.fc2", "1.q_proj"]
+    c = found["1.fc1"]
+    assert (c["k"], c["n"], c["q"], c["num_groups"]) == (64, 128, 3, 2) and c["bW"].shape == (2, 3, 128)
+    assert isinstance(model[0].fc1, torch.nn.Linear)   # untouched
+    with pytest.raises(ValueError, match="no torch.nn.Linear"):
+        Q.quantize_model(torch.nn.Sequential(torch.nn.ReLU()), to_device=False)
+
+
+@pytest.mark.gpu
+def test_quantize_model_on_device(lutgemm, device):
+    """The converted model computes what the same model with the dequantised weights computes:
+    decode-sized inputs take the LUT kernel, larger ones the dense route."""
+    print("case quantize_model", flush=True)
+    from lutgemm.torch_ops import LutLinear
+    torch.manual_seed(9)
+    model = torch.nn.Sequential(_Block(256, 512, True), _Block(256, 512, False)).half().to(device)
+    ref = torch.nn.Sequential(_Block(256, 512, True), _Block(256, 512, False)).half().to(device)
+    ref.load_state_dict(model.state_dict())
+    for blk in ref:
+        for name in ("q_proj", "fc1", "fc2"):
+            lin = getattr(blk, name)
+            _, w_hat = Q.quantize_linear(lin.weight.detach().float(), 4, 64, "rtn")
+            lin.weight.data.copy_(w_hat.half())
+    Q.quantize_model(model, qbits=4, group_size=64, method="rtn")
+    assert all(isinstance(getattr(b, nm), LutLinear) for b in model for nm in ("q_proj", "fc1", "fc2"))
+    assert isinstance(model[0].gate, torch.nn.Linear)
+    for rows in (1, 2, 5, 32):
+        x = torch.randn(rows, 256, device=device, dtype=torch.float16)
+        with torch.no_grad():
+            y, want = model(x), ref(x)
+        err = (y.float() - want.float()).abs().max().item()
+        assert err <= 0.02 * want.float().abs().max().item() + 0.02, (rows, err)
+
+
+@pytest.mark.gpu
+def test_opt_decoder_quantised_end_to_end(lutgemm, device):
+    """A randomly initialised OPT decoder (the model family the reference's walkers convert,
+    examples/quant_model_rtn.py:34): every q/k/v/out projection and both MLP layers replaced by
+    packed weights; prefill and one cached decode step give the logits of the same model run
+    with the dequantised weights."""
+    transformers = pytest.importorskip("transformers")
+    from lutgemm.torch_ops import LutLinear
+    print("case OPT decoder", flush=True)
+    cfg = transformers.OPTConfig(vocab_size=512, hidden_size=256, num_hidden_layers=2, ffn_dim=1024,
+                                 num_attention_heads=4, max_position_embeddings=64, word_embed_proj_dim=256)
+    torch.manual_seed(10)
+    model = transformers.OPTForCausalLM(cfg).eval().half().to(device)
+    ref = transformers.OPTForCausalLM(cfg).eval().half().to(device)
+    ref.load_state_dict(model.state_dict())
+    for name, mod in ref.named_modules():
+        if isinstance(mod, torch.nn.Linear) and any(x in name.split(".")[-1] for x in Q.DEFAULT_LAYERS):
+            _, w_hat = Q.quantize_linear(mod.weight.detach().float(), 4, 128, "rtn")
+            mod.weight.data.copy_(w_hat.half())
+    Q.quantize_model(model, qbits=4, group_size=128, method="rtn")
+    converted = [n for n, m in model.named_modules() if isinstance(m, LutLinear)]
+    assert len(converted) == 12 and isinstance(model.lm_head, torch.nn.Linear)
+    ids = torch.randint(0, 512, (1, 6), device=device)
+    nxt = torch.randint(0, 512, (1, 1), device=device)
+    with torch.no_grad():
+        a = model(ids, use_cache=True)
+        b = ref(ids, use_cache=True)
+        a1 = model(nxt, past_key_values=a.past_key_values, use_cache=True)   # one row: the LUT kernel
+        b1 = ref(nxt, past_key_values=b.past_key_values, use_cache=True)
+        long_ids = torch.randint(0, 512, (2, 12), device=device)             # 24 rows: dense route
+        c, d = model(long_ids).logits, ref(long_ids).logits
+    for got, want, what in ((a.logits, b.logits, "prefill"), (a1.logits, b1.logits, "decode"), (c, d, "batch")):
+        err = (got.float() - want.float()).abs().max().item()
+        assert err <= 0.02 * want.float().abs().max().item() + 0.02, (what, err)
+    assert torch.equal(a1.logits.argmax(-1), b1.logits.argmax(-1))
+
+
 @pytest.mark.gpu
 @pytest.mark.parametrize("method,qbits,g", [("rtn", 4, 128), ("bcq", 3, 128), ("rtn", 3, 64)])
 def test_quantised_linear_on_device(lutgemm, oracle, device, method, qbits, g):
