@@ -35,11 +35,42 @@ __device__ __forceinline__ float scale_from_holder(float v)
     }
 }
 
+// The 8 x 8 weights of outputs P0 .. P0+7 of one half of a batch for this lane's chunk:
+// sgh[b] = the lane's 16 sign bytes of plane b for that half, sch = the GSUB scale slots of that
+// half as held by this lane.  fp32 sum  offset +- alpha_0 +- alpha_1 ...  in plane order.
+template <int Q, bool OFF, int GSUB, int P0>
+__device__ __forceinline__ void expand_step(const u32x4 (&sgh)[Q], const float (&sch)[GSUB * (Q + (OFF ? 1 : 0))],
+                                            float (&w)[8][8])
+{
+    constexpr int QO = Q + (OFF ? 1 : 0);
+    constexpr int SUBL = 16 / GSUB;
+    static_for<8>([&](auto OI) {
+        constexpr int oi = OI;
+        constexpr int ih = P0 + oi;  // output within the half
+        float s[QO];
+#pragma unroll
+        for (int bo = 0; bo < QO; bo++) s[bo] = scale_from_holder<GSUB, ih % SUBL>(sch[(ih / SUBL) * QO + bo]);
+        uint32_t byte[Q];
+#pragma unroll
+        for (int b = 0; b < Q; b++) {
+            const uint32_t word = ih / 4 == 0 ? sgh[b].x : ih / 4 == 1 ? sgh[b].y : ih / 4 == 2 ? sgh[b].z : sgh[b].w;
+            byte[b] = (word >> ((ih % 4) * 8)) & 0xffu;
+        }
+#pragma unroll
+        for (int t = 0; t < 8; t++) {
+            float v = 0.f;
+            if constexpr (OFF) v = s[QO - 1];
+#pragma unroll
+            for (int b = 0; b < Q; b++) v += ((byte[b] >> t) & 1u) ? s[b] : -s[b];
+            w[oi][t] = v;
+        }
+    });
+}
+
 template <int Q, bool OFF, int GSUB>
 __global__ __launch_bounds__(256) void dequantize_kernel(DequantArgs a)
 {
     constexpr int QO = Q + (OFF ? 1 : 0);
-    constexpr int SUBL = 16 / GSUB;
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int nbatches = (a.n + kBatch - 1) / kBatch;
@@ -83,27 +114,7 @@ __global__ __launch_bounds__(256) void dequantize_kernel(DequantArgs a)
         static_for<2>([&](auto P) {
             constexpr int p0 = P * 8;  // outputs h*16 + p0 .. +7: bytes p0 .. p0+7 of the sign vectors
             float w[8][8];             // [output][k]
-            static_for<8>([&](auto OI) {
-                constexpr int oi = OI;
-                constexpr int ih = p0 + oi;  // output within the half
-                float s[QO];
-#pragma unroll
-                for (int bo = 0; bo < QO; bo++) s[bo] = scale_from_holder<GSUB, ih % SUBL>(sch[(ih / SUBL) * QO + bo]);
-                uint32_t byte[Q];
-#pragma unroll
-                for (int b = 0; b < Q; b++) {
-                    const uint32_t word = ih / 4 == 0 ? sgh[b].x : ih / 4 == 1 ? sgh[b].y : ih / 4 == 2 ? sgh[b].z : sgh[b].w;
-                    byte[b] = (word >> ((ih % 4) * 8)) & 0xffu;
-                }
-#pragma unroll
-                for (int t = 0; t < 8; t++) {
-                    float v = 0.f;
-                    if constexpr (OFF) v = s[QO - 1];
-#pragma unroll
-                    for (int b = 0; b < Q; b++) v += ((byte[b] >> t) & 1u) ? s[b] : -s[b];
-                    w[oi][t] = v;
-                }
-            });
+            expand_step<Q, OFF, GSUB, p0>(sgh, sch, w);
             const int col0 = nb * kBatch + h * 16 + p0;  // first of the 8 outputs
 #pragma unroll
             for (int oi = 0; oi < 8; oi++) {
@@ -123,65 +134,93 @@ __global__ __launch_bounds__(256) void dequantize_kernel(DequantArgs a)
     }
 }
 
-// W[k][n], n a multiple of 8: one thread per (chunk, 8 consecutive outputs).  The 64 lanes of a
-// wavefront take 64 consecutive output groups of one chunk, so each of its eight 16-byte stores
-// (one per k of the chunk) writes a 1 KiB run of one row; the four wavefronts of a workgroup take
-// four consecutive chunks, which together use every byte of the 64-byte sign sectors they touch.
-// Sign bytes of 8 outputs are one 8-byte load per plane; scales are 2-byte loads shared through
-// the cache by the lanes of the same k-group.  Same arithmetic and order as the tile kernel.
-__global__ __launch_bounds__(256) void dequantize_rows_kernel(DequantArgs a)
+// W[k][n], n a multiple of 8.  A row of W[k][n] holds the outputs side by side, while a lane of
+// the tile kernel holds 8 k of 8 outputs: written directly, every 16-byte store of a wavefront
+// would go to 64 different rows.  Here a workgroup of eight wavefronts expands two neighbouring
+// batches of one k-block (wavefront = batch x quarter of its outputs, the quarter's sign bytes are
+// one 8-byte load per plane), transposes through LDS and writes whole 128-byte lines: 8 rows x
+// 128 bytes per store instruction.  The LDS image is [512 rows][8 pieces of 16 bytes]; a piece
+// is stored at position (piece ^ (row/8 & 7)) and every 64 rows are followed by 128 bytes of
+// padding, so that 16 consecutive lanes (rows 8 apart) hit 16 different 16-byte bank groups
+// when they write, and the read-back of 8 consecutive rows is one contiguous KiB.
+constexpr int kRowsPitch = 128;                            // bytes per row: 2 batches x 32 outputs x fp16
+constexpr int kRowsLds = kBlockK * kRowsPitch + 8 * 128;   // + padding after every 64 rows
+
+__device__ __forceinline__ int rows_lds_offset(int row, int piece)
 {
-    const int qo = a.q + a.has_offset;
-    const int subl = 16 / a.gsub;
-    const int lh = 2 * a.gsub * qo;
-    const int groups = a.n / 8;
-    const int group_blocks = (groups + 63) / 64;
-    const int og = (int)(blockIdx.x % group_blocks) * 64 + (int)(threadIdx.x & 63);
-    const int c = (int)(blockIdx.x / group_blocks) * 4 + (int)(threadIdx.x >> 6);
-    if (og >= groups || c >= a.k / kChunk) return;
-    const int out0 = og * 8;
-    const int nb = out0 / kBatch, i0 = out0 % kBatch, h = i0 / 16, p0 = i0 % 16;
-    const int ts = c / kLanes, lane = c % kLanes;
-    const size_t tile = (size_t)nb * a.ts + ts;
-    const int r = lane / 16, sub = (lane % 16) / subl;
-    const __half *sc_tile = reinterpret_cast<const __half *>(a.scales) + tile * kLanes * (size_t)lh;
-    // scale record of output i0 + oi: the lane of this k-group that holds it, and the slot in it
-    const __half *sc[8];
+    return row * kRowsPitch + (row >> 6) * 128 + ((piece ^ ((row >> 3) & 7)) << 4);
+}
+
+template <int Q, bool OFF, int GSUB>
+__global__ __launch_bounds__(512) void dequantize_rows_kernel(DequantArgs a)
+{
+    constexpr int QO = Q + (OFF ? 1 : 0);
+    __shared__ __attribute__((aligned(16))) unsigned char image[kRowsLds];
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int nbatches = (a.n + kBatch - 1) / kBatch;
+    const int npairs = (nbatches + 1) / 2;
+    // neighbouring workgroups write neighbouring lines of the same 512 rows
+    const int pair = (int)(blockIdx.x % npairs);
+    const int ts = (int)(blockIdx.x / npairs);
+    const int bi = wave >> 2, st = wave & 3, h = st >> 1;
+    const int nb = pair * 2 + bi;
+
+    if (nb < nbatches) {  // wave-uniform
+        const size_t tile = (size_t)nb * a.ts + ts;
+        const unsigned char *sp =
+            a.signs + (tile * (size_t)(2 * Q) + h) * kUnitBytes + lane * 16 + (st & 1) * 8;
+        const uint32_t *cp = reinterpret_cast<const uint32_t *>(a.scales) + (tile * kLanes + lane) * (size_t)(GSUB * QO);
+        // the 8 sign bytes of this quarter sit in .x/.y (first 8 outputs of the half) or .z/.w
+        u32x4 sgh[Q];
 #pragma unroll
-    for (int oi = 0; oi < 8; oi++) {
-        const int i = i0 + oi;
-        sc[oi] = sc_tile + (size_t)(r * 16 + sub * subl + (i % subl)) * lh + (i / subl) * qo;
-    }
-    float w[8][8];  // [output][k]
+        for (int b = 0; b < Q; b++) {
+            const uint64_t v = __builtin_nontemporal_load(reinterpret_cast<const uint64_t *>(sp + (size_t)(2 * b) * kUnitBytes));
+            sgh[b].x = sgh[b].z = (uint32_t)v;
+            sgh[b].y = sgh[b].w = (uint32_t)(v >> 32);
+        }
+        float sc[2 * GSUB * QO];  // [slot][plane or offset]
 #pragma unroll
-    for (int oi = 0; oi < 8; oi++) {
-        const float off = a.has_offset ? __half2float(sc[oi][a.q]) : 0.f;
+        for (int d = 0; d < GSUB * QO; d++) {
+            const uint32_t rec = __builtin_nontemporal_load(cp + d);
+            const __half2 h2 = *reinterpret_cast<const __half2 *>(&rec);
+            sc[2 * d] = __low2float(h2);
+            sc[2 * d + 1] = __high2float(h2);
+        }
+        float sch[GSUB * QO];  // the GSUB slots of this half
 #pragma unroll
-        for (int t = 0; t < 8; t++) w[oi][t] = off;
-    }
-    const uint8_t *sg = a.signs + (tile * (size_t)(2 * a.q) + h) * kUnitBytes + lane * 16 + p0;
-    for (int b = 0; b < a.q; b++) {
-        const uint64_t bytes = *reinterpret_cast<const uint64_t *>(sg + (size_t)(2 * b) * kUnitBytes);
+        for (int d = 0; d < GSUB * QO; d++) sch[d] = h ? sc[GSUB * QO + d] : sc[d];
+        float w[8][8];  // [output][k]
+        if (st & 1) expand_step<Q, OFF, GSUB, 8>(sgh, sch, w);
+        else        expand_step<Q, OFF, GSUB, 0>(sgh, sch, w);
 #pragma unroll
-        for (int oi = 0; oi < 8; oi++) {
-            const float al = __half2float(sc[oi][b]);
-            const uint32_t byte = (uint32_t)(bytes >> (8 * oi)) & 0xffu;
+        for (int t = 0; t < 8; t++) {
+            __half2 hh[4];
 #pragma unroll
-            for (int t = 0; t < 8; t++) w[oi][t] += ((byte >> t) & 1u) ? al : -al;
+            for (int o2 = 0; o2 < 4; o2++) hh[o2] = __floats2half2_rn(w[2 * o2][t], w[2 * o2 + 1][t]);
+            u32x4 v;
+            v.x = *reinterpret_cast<uint32_t *>(&hh[0]);
+            v.y = *reinterpret_cast<uint32_t *>(&hh[1]);
+            v.z = *reinterpret_cast<uint32_t *>(&hh[2]);
+            v.w = *reinterpret_cast<uint32_t *>(&hh[3]);
+            *reinterpret_cast<u32x4 *>(image + rows_lds_offset(lane * kChunk + t, wave)) = v;
         }
     }
-    __half *dst = reinterpret_cast<__half *>(a.out) + (size_t)c * kChunk * a.n + out0;
+    __syncthreads();
+
+    // 512 threads x 8 rounds: 64 rows x 8 pieces per round, one piece = 8 outputs of one row
+    const int piece = threadIdx.x & 7;
+    const int col = pair * 2 * kBatch + piece * 8;
+    if (col >= a.n) return;  // n is a multiple of 8: a piece is wholly inside or outside
+    __half *dst = reinterpret_cast<__half *>(a.out) + col;
 #pragma unroll
-    for (int t = 0; t < 8; t++) {
-        __half2 hh[4];
-#pragma unroll
-        for (int o2 = 0; o2 < 4; o2++) hh[o2] = __floats2half2_rn(w[2 * o2][t], w[2 * o2 + 1][t]);
-        u32x4 v;
-        v.x = *reinterpret_cast<uint32_t *>(&hh[0]);
-        v.y = *reinterpret_cast<uint32_t *>(&hh[1]);
-        v.z = *reinterpret_cast<uint32_t *>(&hh[2]);
-        v.w = *reinterpret_cast<uint32_t *>(&hh[3]);
-        *reinterpret_cast<u32x4 *>(dst + (size_t)t * a.n) = v;
+    for (int j = 0; j < 8; j++) {
+        const int row = j * 64 + (int)(threadIdx.x >> 3);
+        const int kk = ts * kBlockK + row;
+        if (kk < a.k) {
+            const u32x4 v = *reinterpret_cast<const u32x4 *>(image + rows_lds_offset(row, piece));
+            *reinterpret_cast<u32x4 *>(dst + (size_t)kk * a.n) = v;
+        }
     }
 }
 
@@ -227,10 +266,18 @@ namespace {
 template <int Q, bool OFF>
 hipError_t launch_dequantize_gsub(const DequantArgs &a, unsigned blocks, hipStream_t stream)
 {
-    switch (a.gsub) {
-        case 1: hipLaunchKernelGGL((dequantize_kernel<Q, OFF, 1>), dim3(blocks), dim3(256), 0, stream, a); break;
-        case 2: hipLaunchKernelGGL((dequantize_kernel<Q, OFF, 2>), dim3(blocks), dim3(256), 0, stream, a); break;
-        default: hipLaunchKernelGGL((dequantize_kernel<Q, OFF, 4>), dim3(blocks), dim3(256), 0, stream, a); break;
+    if (a.transposed) {
+        switch (a.gsub) {
+            case 1: hipLaunchKernelGGL((dequantize_kernel<Q, OFF, 1>), dim3(blocks), dim3(256), 0, stream, a); break;
+            case 2: hipLaunchKernelGGL((dequantize_kernel<Q, OFF, 2>), dim3(blocks), dim3(256), 0, stream, a); break;
+            default: hipLaunchKernelGGL((dequantize_kernel<Q, OFF, 4>), dim3(blocks), dim3(256), 0, stream, a); break;
+        }
+    } else {
+        switch (a.gsub) {
+            case 1: hipLaunchKernelGGL((dequantize_rows_kernel<Q, OFF, 1>), dim3(blocks), dim3(512), 0, stream, a); break;
+            case 2: hipLaunchKernelGGL((dequantize_rows_kernel<Q, OFF, 2>), dim3(blocks), dim3(512), 0, stream, a); break;
+            default: hipLaunchKernelGGL((dequantize_rows_kernel<Q, OFF, 4>), dim3(blocks), dim3(512), 0, stream, a); break;
+        }
     }
     return hipGetLastError();
 }
@@ -244,13 +291,7 @@ hipError_t launch_dequantize_q(const DequantArgs &a, unsigned blocks, hipStream_
 
 hipError_t launch_dequantize(const DequantArgs &a, hipStream_t stream)
 {
-    if (!a.transposed && a.n % 8 == 0) {
-        const size_t blocks = (size_t)((a.n / 8 + 63) / 64) * (size_t)(a.k / kChunk / 4);
-        if (blocks > 0x7fffffffu) return hipErrorInvalidValue;
-        hipLaunchKernelGGL(dequantize_rows_kernel, dim3((unsigned)blocks), dim3(256), 0, stream, a);
-        return hipGetLastError();
-    }
-    if (!a.transposed) {
+    if (!a.transposed && a.n % 8 != 0) {
         const size_t total = (size_t)(a.k / kChunk) * (size_t)a.n;
         const size_t blocks = (total + 255) / 256;
         if (blocks > 0x7fffffffu) return hipErrorInvalidValue;
@@ -258,7 +299,7 @@ hipError_t launch_dequantize(const DequantArgs &a, hipStream_t stream)
         return hipGetLastError();
     }
     const size_t nbatches = ((size_t)a.n + kBatch - 1) / kBatch;
-    const size_t blocks = ((nbatches + 3) / 4) * (size_t)a.ts;
+    const size_t blocks = (a.transposed ? (nbatches + 3) / 4 : (nbatches + 1) / 2) * (size_t)a.ts;
     if (blocks > 0x7fffffffu) return hipErrorInvalidValue;
     const unsigned nblk = (unsigned)blocks;
     switch (a.q) {

@@ -239,7 +239,12 @@ def test_back_to_back_launches_reuse_workspace(lutgemm, oracle, device):
 def test_device_round_trip_and_dequantize(lutgemm, oracle, device):
     import torch
     from lutgemm import synth
-    for (k, n, q, g, off) in [(1024, 100, 3, 128, False), (1536, 70, 2, 64, True), (512, 33, 4, 32, True)]:
+    # n % 8 != 0 takes the per-output kernel for W[k][n], n % 8 == 0 the one that writes whole
+    # lines (an odd number of batches leaves half of the last workgroup idle; k = 608 ends inside
+    # a k-block); all three scale layouts (g >= 128, 64, 32) with and without offset
+    for (k, n, q, g, off) in [(1024, 100, 3, 128, False), (1536, 70, 2, 64, True), (512, 33, 4, 32, True),
+                              (1024, 104, 3, 128, False), (1536, 72, 2, 64, True), (608, 40, 4, 32, True),
+                              (2048, 328, 5, 256, True), (640, 8, 1, 64, False), (1024, 512, 8, 32, False)]:
         say("case dequant", k, n, q, g, off)
         w, W = make(lutgemm, synth, k, n, q, g, offset=off, seed=k)
         bW, alpha, z = W.unpack()
