@@ -327,7 +327,7 @@ int run_matvec(const lutgemm_weight *w, const void *x, void *y, int m, void *str
     a.blocks_per_split = w->plan.blocks_per_split;
     const uint16_t *xh = static_cast<const uint16_t *>(x);
     uint16_t *yh = static_cast<uint16_t *>(y);
-    if (((uintptr_t)x & 15u) != 0 || (!cols && m > 1 && (s.k % 8) != 0))
+    if (((uintptr_t)x & 15u) != 0)  // rows of x are k fp16 apart and k is a multiple of 32
         return fail(LUTGEMM_ERR_BAD_SHAPE, "x must be 16-byte aligned");
     hipStream_t st = static_cast<hipStream_t>(stream);
     if (cols && m > 1) {
@@ -408,6 +408,8 @@ int lutgemm_weight_create(const uint32_t *bW, const float *alpha, const float *q
 int lutgemm_weight_clone(const lutgemm_weight *w, lutgemm_weight **out)
 {
     if (!w || !out) return fail(LUTGEMM_ERR_NULL_POINTER, "null argument to weight_clone");
+    *out = nullptr;
+    if (int st_dev = check_device(w)) return st_dev;
     int st = create_from_tiles(w->shape, w->d_signs, w->d_scales, hipMemcpyDeviceToDevice, out);
     if (st == LUTGEMM_OK) (*out)->plan = w->plan;
     return st;
@@ -435,6 +437,7 @@ int lutgemm_weight_save(const lutgemm_weight *w, const char *path)
 int lutgemm_weight_load(const char *path, lutgemm_weight **out)
 {
     if (!path || !out) return fail(LUTGEMM_ERR_NULL_POINTER, "null argument to weight_load");
+    *out = nullptr;
     Shape s;
     std::vector<uint8_t> signs;
     std::vector<uint16_t> scales;
@@ -611,6 +614,7 @@ int lutgemm_weight_set_plan(lutgemm_weight *w, int waves_per_group, int k_splits
 int lutgemm_weight_autotune(lutgemm_weight *w, void *stream)
 {
     if (!w) return fail(LUTGEMM_ERR_NULL_POINTER, "null argument to weight_autotune");
+    if (int st_dev = check_device(w)) return st_dev;
     const Shape &s = w->shape;
     hipStream_t st = static_cast<hipStream_t>(stream);
     // candidates: the best plans of the model, measured on the device
