@@ -211,7 +211,8 @@ def run_single(args, lutgemm, synth, torch, dev, stream, name):
                         "kernel": kernel, "algorithmic_bytes_per_launch": pt.b_total, "avg_launch_us": us}
     line["hot_single_copy"] = {"us_per_matvec": us_hot, "weight_GBps": pt.b_w / (us_hot * 1e-6) / 1e9}
     # the device's pure-read time for the same tiles, same grid, same rotation over the copies
-    lutgemm.read_probe(pt.weights * 3, stream.cuda_stream)
+    # (warmed like the matvec: the device only reaches its sustained clocks under load)
+    lutgemm.read_probe([pt.weights[i % pt.copies] for i in range(max(1, args.warmup))], stream.cuda_stream)
     torch.cuda.synchronize()
     reads = max(1, args.steps)
     order = [pt.weights[i % pt.copies] for i in range(reads)]

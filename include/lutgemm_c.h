@@ -119,9 +119,10 @@ int lutgemm_matvec_many(const lutgemm_weight *const *ws, const void *const *xs, 
 int lutgemm_dequantize(const lutgemm_weight *w, void *d_fW, int transposed, void *stream);
 
 /* Measurement aid without counterpart in the reference: for each of the `count` handles in turn,
- * streams its packed tiles once with a kernel that only reads (same grid as that handle's launch
- * plan, 16-byte loads, nothing written).  The time per launch is the device's pure-read time for
- * the bytes a matvec has to fetch, the ceiling the benchmark quotes next to the matvec.
+ * streams its packed tiles once with a kernel that only reads: the grid of that handle's launch
+ * plan, every wavefront fetching the bytes its matvec wavefront fetches in the same order with
+ * the same number of 16-byte loads in flight, nothing computed or written.  The time per launch
+ * is the device's pure-read time for a matvec's bytes, the floor the benchmark quotes next to it.
  * Asynchronous on `stream`. */
 int lutgemm_read_probe(const lutgemm_weight *const *ws, int count, void *stream);
 

@@ -548,9 +548,18 @@ int lutgemm_read_probe(const lutgemm_weight *const *ws, int count, void *stream)
         if (!w) return fail(LUTGEMM_ERR_NULL_POINTER, "null handle in read_probe");
         if (int st_dev = check_device(w)) return st_dev;
         const Shape &s = w->shape;
-        hipError_t e = lutgemm_kernels::launch_read_probe(w->d_signs, sign_bytes(s), w->d_scales, scale_bytes(s),
-                                                          w->plan.ntiles * w->plan.k_splits, w->plan.waves * kLanes,
-                                                          static_cast<hipStream_t>(stream));
+        lutgemm_kernels::MatvecArgs a{};
+        a.signs = w->d_signs;
+        a.scales = w->d_scales;
+        a.k = s.k;
+        a.n = s.n;
+        a.ts = s.ts;
+        a.nb = s.nb;
+        a.ntiles = w->plan.ntiles;
+        a.k_splits = w->plan.k_splits;
+        a.blocks_per_split = w->plan.blocks_per_split;
+        hipError_t e = lutgemm_kernels::launch_read_probe(s.q, s.has_offset, s.gsub, a, w->plan.ntiles * w->plan.k_splits,
+                                                          w->plan.waves, static_cast<hipStream_t>(stream));
         if (e != hipSuccess) return hip_fail(e, "launch read_probe_kernel");
     }
     return LUTGEMM_OK;

@@ -23,7 +23,7 @@ struct MatvecArgs {
     int y_stride;           // output j goes to y[j * y_stride]
     // rows == 2: a second activation row at x + x_row_stride goes to y + y_row_stride in the
     // same pass (strides in fp16 elements), with its accumulators at accum + accum_row_stride
-    int rows;
+    int rows;               // 1 or 2 activation rows (0 selects the read probe)
     long long x_row_stride, y_row_stride, accum_row_stride;
 };
 
@@ -44,9 +44,10 @@ hipError_t launch_gather_columns(const void *cols, void *rows, int k, int m, hip
 
 hipError_t launch_dequantize(const DequantArgs &a, hipStream_t stream);
 
-// pure read of two byte ranges (multiples of 16 bytes), nothing written
-hipError_t launch_read_probe(const void *a, size_t bytes_a, const void *b, size_t bytes_b, int workgroups,
-                             int threads, hipStream_t stream);
+// The matvec's loads without its arithmetic (same grid and arguments; x, y and accum unused):
+// nothing is written.
+hipError_t launch_read_probe(int q, int has_offset, int gsub, const MatvecArgs &a, int workgroups, int waves,
+                             hipStream_t stream);
 
 }  // namespace lutgemm_kernels
 #endif

@@ -684,34 +684,47 @@ __global__ __launch_bounds__(768) void lut_matvec2_kernel(MatvecArgs a)
     finish_output(total1, active && a.rows > 1, out, lane, y + a.y_row_stride, a.accum + a.accum_row_stride, a);
 }
 
-// Reads two byte ranges once with 16-byte non-temporal loads and does nothing else (the xor of
-// the data only feeds a store that never happens): the time of this kernel over a weight's tiles
-// is the device's pure-read time for the bytes the matvec has to stream.
-__device__ __forceinline__ unsigned read_range(const u32x4 *p, size_t n, size_t tid, size_t stride)
+// The matvec without its arithmetic: same grid, same tile registers, the same loads in the same
+// order refilled at the same points (scale words, then one 16-byte sign vector after the other),
+// the loaded data only xor-ed into a value that is never stored.  No activations, no tables.
+// Its time is the device's pure-read time for the matvec's bytes in the matvec's order.
+template <int Q, bool OFF, int GSUB>
+__global__ __launch_bounds__(768) void read_probe_kernel(MatvecArgs a)
 {
-    constexpr int kInFlight = 6;  // loads per thread before the first use
-    unsigned acc = 0;
-    size_t i = tid;
-    for (; i + (kInFlight - 1) * stride < n; i += kInFlight * stride) {
-        u32x4 v[kInFlight];
-#pragma unroll
-        for (int u = 0; u < kInFlight; u++) v[u] = __builtin_nontemporal_load(p + i + u * stride);
-#pragma unroll
-        for (int u = 0; u < kInFlight; u++) acc ^= v[u].x ^ v[u].y ^ v[u].z ^ v[u].w;
-    }
-    for (; i < n; i += stride) {
-        const u32x4 v = __builtin_nontemporal_load(p + i);
-        acc ^= v.x ^ v.y ^ v.z ^ v.w;
-    }
-    return acc;
-}
+    constexpr int QO = Q + (OFF ? 1 : 0);
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int waves = blockDim.x >> 6;
+    const int ntile = blockIdx.x % a.ntiles;
+    const int ks = blockIdx.x / a.ntiles;
+    const int nb = ntile * waves + wave;
+    const int ts0 = ks * a.blocks_per_split;
+    const int ts1 = min(ts0 + a.blocks_per_split, a.ts);
+    const u32x4 *signs = reinterpret_cast<const u32x4 *>(a.signs);
+    const uint32_t *scales = reinterpret_cast<const uint32_t *>(a.scales);
+    const size_t tile0 = (size_t)(nb < a.nb ? nb : 0) * a.ts;
 
-__global__ __launch_bounds__(768) void read_probe_kernel(const u32x4 *a, size_t na, const u32x4 *b, size_t nb,
-                                                         unsigned *never_written)
-{
-    const size_t tid = (size_t)blockIdx.x * blockDim.x + threadIdx.x, stride = (size_t)gridDim.x * blockDim.x;
-    const unsigned acc = read_range(a, na, tid, stride) ^ read_range(b, nb, tid, stride);
-    if (na + nb == 0 && acc == 0x12345678u) never_written[0] = acc;
+    TileRegs<Q, QO, GSUB> tile;
+    load_tile(tile, tile_address<Q, QO, GSUB>(signs, scales, tile0 + ts0, lane, true));
+    unsigned acc = 0;
+    for (int ts = ts0; ts < ts1; ts++) {
+        const NextTile next = tile_address<Q, QO, GSUB>(signs, scales, tile0 + ts + 1, lane, ts + 1 < ts1);
+#pragma unroll
+        for (int d = 0; d < GSUB * QO; d++) acc ^= tile.scale[d];
+#pragma unroll
+        for (int d = 0; d < GSUB * QO; d++) tile.scale[d] = __builtin_nontemporal_load(next.scale + d);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int u = 0; u < 2 * Q; u++) {
+            // keep each refill right behind the use of its register, as in the matvec
+            acc ^= tile.sign[u].x ^ tile.sign[u].y ^ tile.sign[u].z ^ tile.sign[u].w;
+            tile.sign[u] = __builtin_nontemporal_load(next.sign + u * next.sign_stride);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    }
+#pragma unroll
+    for (int u = 0; u < 2 * Q; u++) acc ^= tile.sign[u].x;  // the dummy loads of the last refill
+    if (a.y && acc == 0x12345678u) *static_cast<unsigned *>(a.y) = acc;
 }
 
 // x [k][m] (m vectors stored as columns) -> rows [m][k], so that the matvec kernel can read
@@ -727,7 +740,9 @@ __global__ __launch_bounds__(256) void gather_columns_kernel(const uint16_t *col
 template <int Q, bool OFF, int GSUB>
 hipError_t launch_one(const MatvecArgs &a, int workgroups, int threads, hipStream_t stream)
 {
-    if (a.rows > 1)
+    if (a.rows == 0)  // read probe
+        hipLaunchKernelGGL((read_probe_kernel<Q, OFF, GSUB>), dim3(workgroups), dim3(threads), 0, stream, a);
+    else if (a.rows > 1)
         hipLaunchKernelGGL((lut_matvec2_kernel<Q, OFF, GSUB>), dim3(workgroups), dim3(threads), 0, stream, a);
     else
     {
@@ -810,13 +825,13 @@ hipError_t launch_gather_columns(const void *cols, void *rows, int k, int m, hip
     return hipGetLastError();
 }
 
-hipError_t launch_read_probe(const void *a, size_t bytes_a, const void *b, size_t bytes_b, int workgroups,
-                             int threads, hipStream_t stream)
+hipError_t launch_read_probe(int q, int has_offset, int gsub, const MatvecArgs &a, int workgroups, int waves,
+                             hipStream_t stream)
 {
-    hipLaunchKernelGGL(read_probe_kernel, dim3(workgroups), dim3(threads), 0, stream,
-                       static_cast<const u32x4 *>(a), bytes_a / 16, static_cast<const u32x4 *>(b), bytes_b / 16,
-                       static_cast<unsigned *>(nullptr));
-    return hipGetLastError();
+    MatvecArgs probe = a;
+    probe.rows = 0;
+    probe.y = nullptr;
+    return launch_matvec(q, has_offset, gsub, probe, workgroups, waves, stream);
 }
 
 }  // namespace lutgemm_kernels
