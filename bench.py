@@ -20,6 +20,8 @@ Other workloads, same protocol, one JSON line each (no CPU / dense legs):
   --config cfg4 [--m M] [--graph]
                               q=2 g=128 decoder layer: QKV, out, FC1, FC2 matvecs back to back,
                               m activation rows; --graph replays the chain from a captured HIP graph
+  --config dequant            dense fp16 weight from the packed tiles (lutgemm_dequantize), both
+                              orientations, cfg1 and cfg2 weights
 """
 import argparse
 import json
@@ -383,13 +385,66 @@ def run_cfg4(args, lutgemm, synth, torch, dev, stream):
     return line
 
 
+def run_dequant(args, lutgemm, synth, torch, dev, stream):
+    """Dense fp16 weight from the packed tiles (the route of batches too large for the LUT
+    kernels): a step is one dequantisation of the cfg1 weight; both orientations and the cfg2
+    weight are reported beside it.  Bytes = packed tiles read + 2 k n written."""
+    import numpy as np
+    from oracle import oracle
+    sh = stream.cuda_stream
+    reps = max(1, min(args.steps, 100))
+    shapes = []
+    for name in ("cfg1", "cfg2"):
+        c = synth.CONFIGS[name]
+        k, n, q, g = c["k"], c["n"], c["q"], c["g"]
+        w = synth.make_weight(k, n, q, g, rtn=c["rtn"], seed=1)
+        W = lutgemm.BCQWeight(w["bW"], w["alpha"], k, n, q, k // g, w["q_bias"])
+        # two outputs alternate so that a launch does not rewrite lines still in the cache
+        outs = [torch.empty((k * n,), dtype=torch.float16, device=dev) for _ in range(2)]
+        rec = {"workload": name, "k": k, "n": n, "q": q, "g": g, "offset": w["q_bias"] is not None}
+        for transposed in (True, False):
+            for i in range(max(4, min(args.warmup, 50))):
+                W.dequantize(outs[i % 2].data_ptr(), transposed, sh)
+            torch.cuda.synchronize()
+
+            def run():
+                for i in range(reps):
+                    W.dequantize(outs[i % 2].data_ptr(), transposed, sh)
+            us = event_time_ms(torch, run, stream) * 1e3 / reps
+            nbytes = 2 * k * n + W.weight_bytes()
+            rec["W[n][k]" if transposed else "W[k][n]"] = {"us": us, "GBps": nbytes / us / 1e3, "bytes": nbytes}
+        # parity of the last result (W[k][n]) on the first 256 outputs against the oracle's dense weight
+        got = outs[(reps - 1) % 2].view(k, n)[:, :256].cpu().numpy().astype(np.float64)
+        z = w["q_bias"].astype(np.float16)[:, :256] if w["q_bias"] is not None else None
+        dense = oracle.dense_weight_f64(np.ascontiguousarray(w["bW"][:, :, :256]),
+                                        np.ascontiguousarray(w["alpha"].astype(np.float16)[:, :, :256]),
+                                        np.ascontiguousarray(z) if z is not None else None)
+        rec["parity"] = {"outputs_checked": 256,
+                         "within_half_ulp_fp16": bool(np.all(np.abs(got - dense) <= 2.0 ** -11 * np.abs(dense) + 2.0 ** -24))}
+        shapes.append(rec)
+        W.close()
+        del outs
+    head = shapes[0]["W[n][k]"]
+    line = base_line(args, "GB/s of dequantisation to dense fp16 (packed tiles read + 2kn written), cfg1 weight, W[n][k]",
+                     head["GBps"], head["us"], "dequantize: cfg1 weight k=n=12288 q=3 g=128 to fp16 W[n][k]", {})
+    line["unit"] = "GB/s (bytes read + written / time)"
+    line["steps"] = reps
+    line["ms_per_step"] = head["us"] / 1e3
+    line["shapes"] = shapes
+    line["roofline"] = {"bound": "hbm", "achieved": head["GBps"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                        "frac": head["GBps"] / HBM_PEAK_GBS, "traffic": None, "kernel": "dequantize_kernel<3,false,1>",
+                        "algorithmic_bytes_per_launch": head["bytes"], "avg_launch_us": head["us"]}
+    line["cpu_baseline"] = None
+    return line
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=400)
     ap.add_argument("--warmup", type=int, default=2000,
                     help="untimed steps first (the device reaches its sustained clocks only after some ms of load)")
-    ap.add_argument("--config", default="cfg1", choices=["cfg0", "cfg1", "cfg2", "cfg3", "cfg4"])
+    ap.add_argument("--config", default="cfg1", choices=["cfg0", "cfg1", "cfg2", "cfg3", "cfg4", "dequant"])
     ap.add_argument("--m", type=int, default=1, help="activation rows (cfg4 only)")
     ap.add_argument("--graph", action="store_true", help="cfg4: also replay the chain from a captured HIP graph")
     ap.add_argument("--copies", type=int, default=17, help="cfg1: distinct weight copies rotated through")
@@ -420,6 +475,8 @@ def main():
         line = run_cfg3(args, lutgemm, synth, torch, dev, stream)
     elif args.config == "cfg4":
         line = run_cfg4(args, lutgemm, synth, torch, dev, stream)
+    elif args.config == "dequant":
+        line = run_dequant(args, lutgemm, synth, torch, dev, stream)
     else:
         line = run_single(args, lutgemm, synth, torch, dev, stream, args.config)
     print(json.dumps(line))
