@@ -291,6 +291,10 @@ def test_random_shapes_plans_and_batches(lutgemm, oracle, device):
         y = run_matvec(lutgemm, W, x, device, cols=bool(case % 2))
         assert_within_tolerance(y, truth_of(oracle, w, x),
                                 "case %d k=%d n=%d q=%d g=%d off=%s m=%d plan=%s" % (case, k, n, q, g, offset, m, W.plan()))
+        if case % 4 == 0:   # the read-only twin of the kernel takes the same plans and shapes
+            import torch
+            lutgemm.read_probe([W, W], torch.cuda.current_stream().cuda_stream)
+            torch.cuda.synchronize()
         W.close()
 
 
