@@ -131,18 +131,21 @@ int lutgemm_read_probe(const lutgemm_weight *const *ws, int count, void *stream)
  * bit patterns; any output pointer may be NULL to skip it.  Synchronous. */
 int lutgemm_weight_unpack(const lutgemm_weight *w, uint32_t *bW, uint16_t *alpha, uint16_t *q_bias);
 
-/* Launch plan chosen for the handle (for benchmarks and tests): workgroup count, waves per
- * workgroup, k-splits and 512-wide k-blocks per workgroup. */
+/* Launch plan of the handle for launches with one activation row (for benchmarks and tests):
+ * workgroup count, waves per workgroup, k-splits and 512-wide k-blocks per workgroup.  Passes
+ * over two rows (m >= 2) have a plan of their own, equal to this one unless
+ * lutgemm_weight_autotune has measured a better one. */
 int lutgemm_weight_plan(const lutgemm_weight *w, int *workgroups, int *waves_per_group,
                         int *k_splits, int *k_blocks_per_group);
 
-/* Override the launch plan (0 keeps the automatic choice for that field); synchronises the
- * device first.  Returns LUTGEMM_ERR_BAD_SHAPE if the request cannot be launched
+/* Override the launch plan, for one-row and two-row launches alike (0 keeps the automatic
+ * choice for that field); synchronises the device first.  Returns LUTGEMM_ERR_BAD_SHAPE if the request cannot be launched
  * (1..12 waves per workgroup, 1..min(k/512 rounded up, 128) k-splits). */
 int lutgemm_weight_set_plan(lutgemm_weight *w, int waves_per_group, int k_splits);
 
 /* Measure the most promising launch plans on the device (a few launches each, on `stream`, with
- * scratch activations of its own) and keep the fastest.  Optional: the automatic plan is chosen
+ * scratch activations of its own) and keep the fastest, separately for launches with one
+ * activation row and for two-row passes.  Optional: the automatic plan is chosen
  * from a model, this replaces it by a measurement.  The measurement streams the weight from
  * HBM as a decoder does: it rotates over temporary device copies of the packed weight (about
  * 1 GiB in total, at most 64 copies) so that no launch finds its weight in the memory-side

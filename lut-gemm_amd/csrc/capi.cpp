@@ -62,7 +62,8 @@ struct lutgemm_weight {
     size_t accum_bytes;
     void *d_xrows;                // staging for column-batched activations, grown on demand
     size_t xrows_bytes;
-    Plan plan;
+    Plan plan;                    // launches with one activation row
+    Plan plan2;                   // passes over two activation rows (m >= 2)
 };
 
 namespace {
@@ -178,7 +179,7 @@ int create_from_tiles(const Shape &s, const void *signs, const void *scales, hip
         if (e != hipSuccess) st = hip_fail(e, "hipMemcpy(scales)");
     }
     if (st == LUTGEMM_OK) {
-        w->plan = choose_plan(s, w->compute_units);
+        w->plan = w->plan2 = choose_plan(s, w->compute_units);
         st = alloc_workspace(w);
     }
     if (st != LUTGEMM_OK) {
@@ -322,9 +323,6 @@ int run_matvec(const lutgemm_weight *w, const void *x, void *y, int m, void *str
     a.n = s.n;
     a.ts = s.ts;
     a.nb = s.nb;
-    a.ntiles = w->plan.ntiles;
-    a.k_splits = w->plan.k_splits;
-    a.blocks_per_split = w->plan.blocks_per_split;
     const uint16_t *xh = static_cast<const uint16_t *>(x);
     uint16_t *yh = static_cast<uint16_t *>(y);
     if (((uintptr_t)x & 15u) != 0)  // rows of x are k fp16 apart and k is a multiple of 32
@@ -353,6 +351,10 @@ int run_matvec(const lutgemm_weight *w, const void *x, void *y, int m, void *str
     a.accum_row_stride = (long long)s.nb * kBatch;
     for (int r = 0; r < m; r += 2) {
         a.rows = m - r >= 2 ? 2 : 1;
+        const Plan &plan = a.rows == 2 ? w->plan2 : w->plan;
+        a.ntiles = plan.ntiles;
+        a.k_splits = plan.k_splits;
+        a.blocks_per_split = plan.blocks_per_split;
         a.x = xh + (size_t)r * s.k;
         if (cols) {  // y [n][m]
             a.y = yh + r;
@@ -363,8 +365,8 @@ int run_matvec(const lutgemm_weight *w, const void *x, void *y, int m, void *str
             a.y_stride = 1;
             a.y_row_stride = s.n;
         }
-        hipError_t e = lutgemm_kernels::launch_matvec(s.q, s.has_offset, s.gsub, a,
-                                                      w->plan.ntiles * w->plan.k_splits, w->plan.waves, st);
+        hipError_t e = lutgemm_kernels::launch_matvec(s.q, s.has_offset, s.gsub, a, plan.ntiles * plan.k_splits,
+                                                      plan.waves, st);
         if (e != hipSuccess) return hip_fail(e, "launch lut_matvec_kernel");
     }
     return LUTGEMM_OK;
@@ -411,7 +413,10 @@ int lutgemm_weight_clone(const lutgemm_weight *w, lutgemm_weight **out)
     *out = nullptr;
     if (int st_dev = check_device(w)) return st_dev;
     int st = create_from_tiles(w->shape, w->d_signs, w->d_scales, hipMemcpyDeviceToDevice, out);
-    if (st == LUTGEMM_OK) (*out)->plan = w->plan;
+    if (st == LUTGEMM_OK) {
+        (*out)->plan = w->plan;
+        (*out)->plan2 = w->plan2;
+    }
     return st;
 }
 
@@ -616,7 +621,7 @@ int lutgemm_weight_set_plan(lutgemm_weight *w, int waves_per_group, int k_splits
     }
     hipError_t e = hipDeviceSynchronize();  // no launch may still be using the old workspace
     if (e != hipSuccess) return hip_fail(e, "hipDeviceSynchronize");
-    w->plan = p;
+    w->plan = w->plan2 = p;
     return alloc_workspace(w);
 }
 
@@ -666,24 +671,24 @@ int lutgemm_weight_autotune(lutgemm_weight *w, void *stream)
     void *x = nullptr, *y = nullptr;
     hipEvent_t e0 = nullptr, e1 = nullptr;
     int status = LUTGEMM_OK;
-    hipError_t e = hipMalloc(&x, (size_t)s.k * 2);
-    if (e == hipSuccess) e = hipMalloc(&y, (size_t)s.n * 2);
-    if (e == hipSuccess) e = hipMemsetAsync(x, 0, (size_t)s.k * 2, st);
+    hipError_t e = hipMalloc(&x, (size_t)2 * s.k * 2);
+    if (e == hipSuccess) e = hipMalloc(&y, (size_t)2 * s.n * 2);
+    if (e == hipSuccess) e = hipMemsetAsync(x, 0, (size_t)2 * s.k * 2, st);
     if (e == hipSuccess) e = hipEventCreate(&e0);
     if (e == hipSuccess) e = hipEventCreate(&e1);
     if (e != hipSuccess) status = hip_fail(e, "autotune setup");
-    const Plan before = w->plan;
+    const Plan before = w->plan, before2 = w->plan2;
     size_t turn = 0;
-    // time `reps` launches of plan p rotating over the copies
-    auto measure = [&](const Plan &p, int reps, float *ms_out) -> int {
-        for (lutgemm_weight *c : copies) c->plan = p;
+    // time `reps` launches over `rows` activation rows with plan p, rotating over the copies
+    auto measure = [&](const Plan &p, int rows, int reps, float *ms_out) -> int {
+        for (lutgemm_weight *c : copies) (rows == 2 ? c->plan2 : c->plan) = p;
         int stt = LUTGEMM_OK;
         for (int r = 0; r < 2 && stt == LUTGEMM_OK; r++)
-            stt = run_matvec(copies[turn++ % copies.size()], x, y, 1, stream, false);
+            stt = run_matvec(copies[turn++ % copies.size()], x, y, rows, stream, false);
         if (stt != LUTGEMM_OK) return stt;
         hipError_t he = hipEventRecord(e0, st);
         for (int r = 0; r < reps && stt == LUTGEMM_OK; r++)
-            stt = run_matvec(copies[turn++ % copies.size()], x, y, 1, stream, false);
+            stt = run_matvec(copies[turn++ % copies.size()], x, y, rows, stream, false);
         if (stt != LUTGEMM_OK) return stt;
         if (he == hipSuccess) he = hipEventRecord(e1, st);
         if (he == hipSuccess) he = hipEventSynchronize(e1);
@@ -699,32 +704,36 @@ int lutgemm_weight_autotune(lutgemm_weight *w, void *stream)
         float ms = 0.f;
         while (status == LUTGEMM_OK &&
                std::chrono::duration<double>(std::chrono::steady_clock::now() - t0).count() < 0.03)
-            status = measure(before, 50, &ms);
+            status = measure(before, 1, 50, &ms);
     }
-    // two sweeps over all candidates (the minimum of the two counts), then the four best
-    // again with more launches
-    struct Timed { float ms; Plan p; };
-    std::vector<Timed> timed;
-    for (size_t i = 0; status == LUTGEMM_OK && i < cands.size(); i++) timed.push_back(Timed{1e30f, cands[i].p});
-    for (int sweep = 0; sweep < 2; sweep++)
-        for (size_t i = 0; status == LUTGEMM_OK && i < timed.size(); i++) {
-            float ms = 0.f;
-            status = measure(timed[i].p, 12, &ms);
-            if (status == LUTGEMM_OK && ms < timed[i].ms) timed[i].ms = ms;
-        }
-    std::sort(timed.begin(), timed.end(), [](const Timed &a, const Timed &b) { return a.ms < b.ms; });
-    Plan best = before;
-    float best_ms = 1e30f;
-    for (int round = 0; round < 2; round++)
-        for (size_t i = 0; status == LUTGEMM_OK && i < timed.size() && i < 4; i++) {
-            float ms = 0.f;
-            status = measure(timed[i].p, 50, &ms);
-            if (status == LUTGEMM_OK && ms < best_ms) {
-                best_ms = ms;
-                best = timed[i].p;
+    // Once for launches with one activation row, once for the two-row passes (a different
+    // kernel with its own balance of table building and lookups).  Each time: two sweeps over all
+    // candidates (the minimum of the two counts), then the four best again with more launches.
+    Plan chosen[2] = {before, before2};
+    for (int rows = 1; rows <= 2; rows++) {
+        struct Timed { float ms; Plan p; };
+        std::vector<Timed> timed;
+        for (size_t i = 0; status == LUTGEMM_OK && i < cands.size(); i++) timed.push_back(Timed{1e30f, cands[i].p});
+        for (int sweep = 0; sweep < 2; sweep++)
+            for (size_t i = 0; status == LUTGEMM_OK && i < timed.size(); i++) {
+                float ms = 0.f;
+                status = measure(timed[i].p, rows, 12, &ms);
+                if (status == LUTGEMM_OK && ms < timed[i].ms) timed[i].ms = ms;
             }
-        }
-    w->plan = status == LUTGEMM_OK ? best : before;
+        std::sort(timed.begin(), timed.end(), [](const Timed &a, const Timed &b) { return a.ms < b.ms; });
+        float best_ms = 1e30f;
+        for (int round = 0; round < 2; round++)
+            for (size_t i = 0; status == LUTGEMM_OK && i < timed.size() && i < 4; i++) {
+                float ms = 0.f;
+                status = measure(timed[i].p, rows, 50, &ms);
+                if (status == LUTGEMM_OK && ms < best_ms) {
+                    best_ms = ms;
+                    chosen[rows - 1] = timed[i].p;
+                }
+            }
+    }
+    w->plan = status == LUTGEMM_OK ? chosen[0] : before;
+    w->plan2 = status == LUTGEMM_OK ? chosen[1] : before2;
     if (e0) (void)hipEventDestroy(e0);
     if (e1) (void)hipEventDestroy(e1);
     if (x) (void)hipFree(x);
