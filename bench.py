@@ -265,6 +265,19 @@ def run_single(args, lutgemm, synth, torch, dev, stream, name):
                  "bytes": 2 * k * n + 2 * k + 2 * n,
                  "GBps": (2 * k * n + 2 * k + 2 * n) / (dense_us * 1e-6) / 1e9,
                  "lut_speedup": dense_us / us}
+        # the same product through this library's plain streaming kernel (bandwidth-bound comparator)
+        sh = stream.cuda_stream
+        for i in range(10):
+            lutgemm.dense_gemv(Wd[i % nd].data_ptr(), xv.data_ptr(), outs[i % nd].data_ptr(), k, n, sh)
+        torch.cuda.synchronize()
+        agree = bool(torch.allclose(outs[9 % nd].float(), torch.mv(Wd[9 % nd], xv).float(), rtol=2e-2, atol=2e-2))
+
+        def run_plain():
+            for i in range(reps):
+                lutgemm.dense_gemv(Wd[i % nd].data_ptr(), xv.data_ptr(), outs[i % nd].data_ptr(), k, n, sh)
+        pus = event_time_ms(torch, run_plain, stream) * 1e3 / reps
+        dense["handwritten_streaming_gemv"] = {"us_per_matvec": pus, "GBps": dense["bytes"] / pus / 1e3,
+                                                "lut_speedup": pus / us, "agrees_with_library": agree}
         del Wd
     line["dense_fp16_gemv"] = dense
     line["cpu_baseline"] = None

@@ -126,6 +126,13 @@ int lutgemm_dequantize(const lutgemm_weight *w, void *d_fW, int transposed, void
  * Asynchronous on `stream`. */
 int lutgemm_read_probe(const lutgemm_weight *const *ws, int count, void *stream);
 
+/* Comparator without counterpart in the reference's library (its test times cuBLAS next to the
+ * LUT kernel, tests/opt/fp16/int3_col_wise_matmul_fp16.cu:302-313): a plain bandwidth-bound dense
+ * fp16 matrix-vector product y[n] = sum_k W[n][k] x[k] for a dense weight stored as W^T [n][k]
+ * (the layout lutgemm_dequantize writes with transposed = 1), fp32 accumulation, fp16 result.
+ * k a multiple of 8; d_wt and d_x 16-byte aligned device pointers.  Asynchronous on `stream`. */
+int lutgemm_dense_gemv_f16(const void *d_wt, const void *d_x, void *d_y, int k, int n, void *stream);
+
 /* Copy the packed planes back into the host input layout (exact inverse of the re-tiling):
  * bW [k/32][q][n] uint32, alpha [num_groups][q][n] and q_bias [num_groups][n] as binary16
  * bit patterns; any output pointer may be NULL to skip it.  Synchronous. */

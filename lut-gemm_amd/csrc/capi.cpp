@@ -570,6 +570,24 @@ int lutgemm_read_probe(const lutgemm_weight *const *ws, int count, void *stream)
     return LUTGEMM_OK;
 }
 
+int lutgemm_dense_gemv_f16(const void *d_wt, const void *d_x, void *d_y, int k, int n, void *stream)
+{
+    if (!d_wt || !d_x || !d_y) return fail(LUTGEMM_ERR_NULL_POINTER, "null argument to dense_gemv_f16");
+    if (k < 8 || k % 8 != 0 || n < 1)
+        return fail(LUTGEMM_ERR_BAD_SHAPE, "dense_gemv_f16 needs k a positive multiple of 8 and n >= 1 (k=%d n=%d)", k, n);
+    if ((((uintptr_t)d_wt | (uintptr_t)d_x) & 15u) != 0)
+        return fail(LUTGEMM_ERR_BAD_SHAPE, "dense_gemv_f16 needs 16-byte aligned weight and activations");
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return hip_fail(e, "hipGetDevice");
+    int cus = 0;
+    e = hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);
+    if (e != hipSuccess) return hip_fail(e, "hipDeviceGetAttribute");
+    e = lutgemm_kernels::launch_dense_gemv(d_wt, d_x, d_y, k, n, cus > 0 ? cus : 256, static_cast<hipStream_t>(stream));
+    if (e != hipSuccess) return hip_fail(e, "launch dense_gemv_kernel");
+    return LUTGEMM_OK;
+}
+
 int lutgemm_weight_unpack(const lutgemm_weight *w, uint32_t *bW, uint16_t *alpha, uint16_t *q_bias)
 {
     if (!w) return fail(LUTGEMM_ERR_NULL_POINTER, "null argument to weight_unpack");

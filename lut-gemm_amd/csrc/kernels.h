@@ -49,5 +49,9 @@ hipError_t launch_dequantize(const DequantArgs &a, hipStream_t stream);
 hipError_t launch_read_probe(int q, int has_offset, int gsub, const MatvecArgs &a, int workgroups, int waves,
                              hipStream_t stream);
 
+// Dense fp16 comparator: y[n] = sum_k W^T[n][k] x[k]; k a multiple of 8, pointers 16-byte aligned.
+hipError_t launch_dense_gemv(const void *wt, const void *x, void *y, int k, int n, int compute_units,
+                             hipStream_t stream);
+
 }  // namespace lutgemm_kernels
 #endif

@@ -30,7 +30,7 @@ EXPORTED = [
     "lutgemm_weight_plan", "lutgemm_weight_set_plan", "lutgemm_weight_autotune", "lutgemm_weight_device_ptrs", "lutgemm_packed_sizes",
     "lutgemm_pack_host", "lutgemm_unpack_host", "lutgemm_float_to_half", "lutgemm_last_error",
     "lutgemm_status_string", "lutgemm_version", "lutgemm_pack_file", "lutgemm_unpack_file", "lutgemm_weight_save",
-    "lutgemm_weight_load", "lutgemm_weight_clone", "lutgemm_read_probe",
+    "lutgemm_weight_load", "lutgemm_weight_clone", "lutgemm_read_probe", "lutgemm_dense_gemv_f16",
 ]
 
 
@@ -88,6 +88,7 @@ def load():
     L.lutgemm_weight_load.argtypes = [ctypes.c_char_p, pp]
     L.lutgemm_weight_clone.argtypes = [vp, pp]
     L.lutgemm_read_probe.argtypes = [vp, i, vp]
+    L.lutgemm_dense_gemv_f16.argtypes = [vp, vp, vp, i, i, vp]
     L.lutgemm_weight_set_plan.argtypes = [vp, i, i]
     L.lutgemm_weight_autotune.argtypes = [vp, vp]
     L.lutgemm_weight_device_ptrs.argtypes = [vp, pp, pp, pp]
@@ -313,6 +314,12 @@ def read_probe(weights, stream=0):
     """Pure read of the packed tiles of each weight in turn (measurement aid), one C call."""
     arr = (ctypes.c_void_p * len(weights))(*[w._h for w in weights])
     _check(load().lutgemm_read_probe(arr, len(weights), stream or None))
+
+
+def dense_gemv(wt_ptr, x_ptr, y_ptr, k, n, stream=0):
+    """Comparator: y[n] = sum_k W^T[n][k] x[k] for a dense fp16 weight on the device (device
+    pointers as integers)."""
+    _check(load().lutgemm_dense_gemv_f16(wt_ptr, x_ptr, y_ptr, k, n, stream or None))
 
 
 def version():

@@ -127,6 +127,10 @@ def test_file_entry_points_check_their_arguments(lutgemm, tmp_path):
     assert L.lutgemm_read_probe(None, 1, None) == lutgemm.ERR_NULL_POINTER
     assert L.lutgemm_read_probe((ctypes.c_void_p * 1)(None), 1, None) == lutgemm.ERR_NULL_POINTER
     assert L.lutgemm_read_probe((ctypes.c_void_p * 1)(None), 0, None) == lutgemm.OK
+    buf = (ctypes.c_uint16 * 64)()
+    assert L.lutgemm_dense_gemv_f16(None, buf, buf, 64, 1, None) == lutgemm.ERR_NULL_POINTER
+    assert L.lutgemm_dense_gemv_f16(buf, buf, buf, 60, 1, None) == lutgemm.ERR_BAD_SHAPE
+    assert L.lutgemm_dense_gemv_f16(buf, buf, buf, 64, 0, None) == lutgemm.ERR_BAD_SHAPE
     assert L.lutgemm_status_string(lutgemm.ERR_IO) == b"file input/output failed"
     assert h.value is None
     if not torch.cuda.is_available():

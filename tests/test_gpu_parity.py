@@ -325,3 +325,24 @@ def test_non_finite_activations(lutgemm, device):
         assert np.array_equal(again.view(np.uint16), clean.view(np.uint16))
     W.close()
 
+
+
+def test_dense_gemv_comparator(lutgemm, device):
+    """The plain streaming fp16 GEMV that the benchmark times next to the LUT kernel: fp32
+    accumulation over fp16 inputs, rows whose length is not a multiple of the unrolled step, more
+    rows than wavefronts and fewer."""
+    import torch
+    rng = np.random.default_rng(77)
+    st = torch.cuda.current_stream().cuda_stream
+    for (k, n) in [(8, 1), (328, 37), (4096, 5000), (12288, 70), (520, 4099)]:
+        say("case dense gemv", k, n)
+        W = (rng.standard_normal((n, k)) * 0.05).astype(np.float16)
+        x = rng.standard_normal(k).astype(np.float16)
+        Wd, xd = torch.from_numpy(W).to(device), torch.from_numpy(x).to(device)
+        yd = torch.full((n,), float("nan"), dtype=torch.float16, device=device)
+        lutgemm.dense_gemv(Wd.data_ptr(), xd.data_ptr(), yd.data_ptr(), k, n, st)
+        torch.cuda.synchronize()
+        truth = W.astype(np.float64) @ x.astype(np.float64)
+        got = yd.cpu().numpy().astype(np.float64)
+        # one fp16 rounding of the result plus fp32 accumulation error
+        assert np.all(np.abs(got - truth) <= 2.0 ** -10 * np.abs(truth) + 1e-3), (k, n, np.abs(got - truth).max())
