@@ -41,7 +41,8 @@ METRIC = "µs/matvec + weight-GB/s (% HBM peak), n=k=12288 q=3 g=128 m=1 fp16"
 # HBM bytes per cfg1 launch from the rocprofv3 counter runs summarised in
 # profiles/lut_matvec_kernel_cfg1.md (FETCH_SIZE and WRITE_SIZE, scaled by the factors a plain
 # copy kernel of known size reads on the same counters)
-CFG1_MEASURED_TRAFFIC_BYTES = 64.9e6  # plan 12 waves x 8 k-splits; 64.6e6 with 5 k-splits (fewer atomics)
+# (64.01 MB read for either plan; 0.91 MB written with 8 k-splits, 0.61 MB with 5: fewer split-k atomics)
+CFG1_MEASURED_TRAFFIC_BYTES = {8: 64.9e6, 5: 64.6e6}  # by k-splits of the launch plan
 
 
 def event_time_ms(torch, fn, stream):
@@ -209,7 +210,7 @@ def run_single(args, lutgemm, synth, torch, dev, stream, name):
     kernel = "lut_matvec_kernel<%d,%s,1>" % (q, "true" if pt.has_offset else "false")
     line["roofline"] = {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                         "frac": achieved / HBM_PEAK_GBS,
-                        "traffic": CFG1_MEASURED_TRAFFIC_BYTES if name == "cfg1" else None,
+                        "traffic": CFG1_MEASURED_TRAFFIC_BYTES.get(pt.plan["k_splits"]) if name == "cfg1" else None,
                         "kernel": kernel, "algorithmic_bytes_per_launch": pt.b_total, "avg_launch_us": us}
     line["hot_single_copy"] = {"us_per_matvec": us_hot, "weight_GBps": pt.b_w / (us_hot * 1e-6) / 1e9}
     # the device's pure-read time for the same tiles, same grid, same rotation over the copies
