@@ -5,6 +5,8 @@ CUDA device, so each function is pinned by what the mathematics fixes: the unifo
 of examples/rtn_parameter.py:77-96 checked exhaustively, exact recovery of weights that are
 representable, the greedy closed form of examples/bcq.py:105-119, monotone error under
 refinement, and agreement of the packed container with the dense weight the oracle rebuilds."""
+import os
+
 import numpy as np
 import pytest
 import torch
@@ -313,6 +315,33 @@ def test_quantize_model_finds_the_projection_layers():
     assert isinstance(model[0].fc1, torch.nn.Linear)   # untouched
     with pytest.raises(ValueError, match="no torch.nn.Linear"):
         Q.quantize_model(torch.nn.Sequential(torch.nn.ReLU()), to_device=False)
+
+
+def test_quant_model_cli_writes_loadable_files(tmp_path, lutgemm, oracle):
+    """python -m lutgemm.quant_model, the counterpart of examples/quant_model_rtn.py: a randomly
+    initialised OPT saved locally goes in, one packed file per projection layer comes out, and
+    a file holds the quantised layer (checked against the oracle's dense weight)."""
+    transformers = pytest.importorskip("transformers")
+    from lutgemm import quant_model
+    cfg = transformers.OPTConfig(vocab_size=64, hidden_size=64, num_hidden_layers=1, ffn_dim=128,
+                                 num_attention_heads=2, max_position_embeddings=16, word_embed_proj_dim=64)
+    torch.manual_seed(11)
+    model = transformers.OPTForCausalLM(cfg)
+    src, out = tmp_path / "opt-tiny", tmp_path / "packed"
+    model.save_pretrained(src)
+    assert quant_model.main(["--model_name_or_path", str(src), "--qbits", "3", "--group_size", "32",
+                             "--method", "rtn", "--out_dir", str(out)]) == 0
+    files = sorted(f for f in os.listdir(out) if f.endswith(".lutw"))
+    assert len(files) == 6 and "model.decoder.layers.0.fc1.lutw" in files
+    assert os.path.exists(out / "model.decoder.layers.0.fc1.bias.npy")
+    f = lutgemm.unpack_file(str(out / "model.decoder.layers.0.fc1.lutw"))
+    assert (f["k"], f["n"], f["q"], f["num_groups"]) == (64, 128, 3, 2) and f["q_bias"] is not None
+    w = model.model.decoder.layers[0].fc1.weight.detach().float()
+    _, w_hat = Q.quantize_linear(w, 3, 32, "rtn")
+    dense = oracle.dense_weight_f64(f["bW"], f["alpha"], f["q_bias"])          # [k][n]
+    assert np.abs(dense.T - w_hat.numpy()).max() <= 2e-3 * np.abs(w_hat.numpy()).max() + 1e-4
+    with pytest.raises(SystemExit):
+        quant_model.main(["--model_name_or_path", str(tmp_path / "missing"), "--out_dir", str(out)])
 
 
 @pytest.mark.gpu
