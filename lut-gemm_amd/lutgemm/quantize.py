@@ -379,3 +379,33 @@ def quantize_model(model, qbits=4, group_size=128, method="rtn", rounds=15, laye
     if not found:
         raise ValueError("no torch.nn.Linear child matches %s" % (tuple(layers),))
     return model if to_device else found
+
+
+def load_packed_model(model, directory, layers=DEFAULT_LAYERS, **layer_kw):
+    """Replace every torch.nn.Linear child whose name contains one of `layers` and for which
+    <directory>/<qualified name>.lutw exists (as `python -m lutgemm.quant_model` writes them) by
+    a LutLinear read from that file on the current GPU; the layer keeps its bias.  Returns the
+    list of replaced layer names; raises if no file matches."""
+    import os
+
+    from .torch_ops import LutLinear
+    done = []
+
+    def walk(module, prefix):
+        for name, child in list(module.named_children()):
+            full = prefix + name
+            walk(child, full + ".")
+            path = os.path.join(directory, full + ".lutw")
+            if isinstance(child, torch.nn.Linear) and any(x in name for x in layers) and os.path.exists(path):
+                bias = None if child.bias is None else child.bias.detach()
+                lut = LutLinear.from_file(path, bias=bias, **layer_kw)
+                if (lut.in_features, lut.out_features) != (child.in_features, child.out_features):
+                    raise ValueError("%s holds a %dx%d weight, layer %s is %dx%d" % (
+                        path, lut.in_features, lut.out_features, full, child.in_features, child.out_features))
+                setattr(module, name, lut)
+                done.append(full)
+
+    walk(model, "")
+    if not done:
+        raise ValueError("no packed-weight file in %s matches a layer of the model" % directory)
+    return done

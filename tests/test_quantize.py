@@ -345,6 +345,34 @@ def test_quant_model_cli_writes_loadable_files(tmp_path, lutgemm, oracle):
 
 
 @pytest.mark.gpu
+def test_packed_files_load_into_a_model(tmp_path, lutgemm, device):
+    """Offline packing, then loading: the model read from the files computes exactly what the
+    model built from the same containers in memory computes."""
+    print("case load_packed_model", flush=True)
+    torch.manual_seed(12)
+    base = torch.nn.Sequential(_Block(256, 512, True), _Block(256, 512, False)).half().float()  # fp16-exact weights
+    found = Q.quantize_model(base, qbits=3, group_size=128, method="rtn", to_device=False)
+    for name, c in found.items():
+        lutgemm.pack_file(str(tmp_path / (name + ".lutw")), c["bW"], c["alpha"], c["k"], c["n"], c["q"],
+                          c["num_groups"], c["q_bias"])
+    import copy
+    a = copy.deepcopy(base).half().to(device)
+    b = copy.deepcopy(base).half().to(device)
+    from lutgemm.torch_ops import LutLinear
+    for name, c in found.items():     # the same containers, straight from memory
+        blk, attr = name.split(".")
+        lin = getattr(a[int(blk)], attr)
+        setattr(a[int(blk)], attr, LutLinear(c, bias=None if lin.bias is None else lin.bias.detach()))
+    names = Q.load_packed_model(b, str(tmp_path))
+    assert sorted(names) == sorted(found)
+    x = torch.randn(3, 256, device=device, dtype=torch.float16)
+    with torch.no_grad():
+        assert torch.equal(a(x), b(x))
+    with pytest.raises(ValueError, match="no packed-weight file"):
+        Q.load_packed_model(copy.deepcopy(base), str(tmp_path / "nothing-here"))
+
+
+@pytest.mark.gpu
 def test_quantize_model_on_device(lutgemm, device):
     """The converted model computes what the same model with the dequantised weights computes:
     decode-sized inputs take the LUT kernel, larger ones the dense route."""
