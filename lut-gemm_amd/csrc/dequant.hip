@@ -12,14 +12,14 @@ using namespace lutgemm_layout;
 namespace {
 
 // ------------------------------------------------------------------------------------------
-// Dense fp16 weight from the packed tiles: W[k][n] or W[n][k], offset included.
+// dequantize_kernel: dense fp16 weight W^T [n][k] from the packed tiles, offset included.
 // One wavefront per tile (32 outputs x 512 k), lane L on chunk L as in the matvec: 2q coalesced
 // 16-byte sign loads and one scale record per lane, scales fetched across lanes with DPP, then
 // per weight the fp32 sum  offset +- alpha_0 +- alpha_1 ...  in plane order (the order of
 // lutGEMM::dequantize_cpu, lutGEMM/src/nQWeight_fp16.cu:38-59, so offset-free results are
 // bit-identical to it), one rounding to fp16, 16-byte stores: 8 consecutive k of one output
 // (a wavefront writes 1 KiB runs of a row of W[n][k]).  A workgroup is four wavefronts on four
-// neighbouring batches of the same k-block.  Writes W[n][k].
+// neighbouring batches of the same k-block.  (dequantize_rows_kernel below writes W[k][n].)
 // ------------------------------------------------------------------------------------------
 template <int GSUB, int LANE_IN_SUB>
 __device__ __forceinline__ float scale_from_holder(float v)
