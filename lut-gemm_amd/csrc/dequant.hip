@@ -303,30 +303,14 @@ hipError_t launch_dequantize(const DequantArgs &a, hipStream_t stream)
     if (blocks > 0x7fffffffu) return hipErrorInvalidValue;
     const unsigned nblk = (unsigned)blocks;
     switch (a.q) {
-#if !defined(LUTGEMM_DEV_ONLY_Q) || LUTGEMM_DEV_ONLY_Q == 1
         case 1: return launch_dequantize_q<1>(a, nblk, stream);
-#endif
-#if !defined(LUTGEMM_DEV_ONLY_Q) || LUTGEMM_DEV_ONLY_Q == 2
         case 2: return launch_dequantize_q<2>(a, nblk, stream);
-#endif
-#if !defined(LUTGEMM_DEV_ONLY_Q) || LUTGEMM_DEV_ONLY_Q == 3
         case 3: return launch_dequantize_q<3>(a, nblk, stream);
-#endif
-#if !defined(LUTGEMM_DEV_ONLY_Q) || LUTGEMM_DEV_ONLY_Q == 4
         case 4: return launch_dequantize_q<4>(a, nblk, stream);
-#endif
-#if !defined(LUTGEMM_DEV_ONLY_Q) || LUTGEMM_DEV_ONLY_Q == 5
         case 5: return launch_dequantize_q<5>(a, nblk, stream);
-#endif
-#if !defined(LUTGEMM_DEV_ONLY_Q) || LUTGEMM_DEV_ONLY_Q == 6
         case 6: return launch_dequantize_q<6>(a, nblk, stream);
-#endif
-#if !defined(LUTGEMM_DEV_ONLY_Q) || LUTGEMM_DEV_ONLY_Q == 7
         case 7: return launch_dequantize_q<7>(a, nblk, stream);
-#endif
-#if !defined(LUTGEMM_DEV_ONLY_Q) || LUTGEMM_DEV_ONLY_Q == 8
         case 8: return launch_dequantize_q<8>(a, nblk, stream);
-#endif
         default: return hipErrorInvalidValue;
     }
 }

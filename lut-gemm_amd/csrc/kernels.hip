@@ -820,30 +820,14 @@ hipError_t launch_matvec(int q, int has_offset, int gsub, const MatvecArgs &a, i
 {
     const int th = waves * kLanes;
     switch (q) {
-#if !defined(LUTGEMM_DEV_ONLY_Q) || LUTGEMM_DEV_ONLY_Q == 1
         case 1: return launch_off<1>(has_offset, gsub, a, workgroups, th, stream);
-#endif
-#if !defined(LUTGEMM_DEV_ONLY_Q) || LUTGEMM_DEV_ONLY_Q == 2
         case 2: return launch_off<2>(has_offset, gsub, a, workgroups, th, stream);
-#endif
-#if !defined(LUTGEMM_DEV_ONLY_Q) || LUTGEMM_DEV_ONLY_Q == 3
         case 3: return launch_off<3>(has_offset, gsub, a, workgroups, th, stream);
-#endif
-#if !defined(LUTGEMM_DEV_ONLY_Q) || LUTGEMM_DEV_ONLY_Q == 4
         case 4: return launch_off<4>(has_offset, gsub, a, workgroups, th, stream);
-#endif
-#if !defined(LUTGEMM_DEV_ONLY_Q) || LUTGEMM_DEV_ONLY_Q == 5
         case 5: return launch_off<5>(has_offset, gsub, a, workgroups, th, stream);
-#endif
-#if !defined(LUTGEMM_DEV_ONLY_Q) || LUTGEMM_DEV_ONLY_Q == 6
         case 6: return launch_off<6>(has_offset, gsub, a, workgroups, th, stream);
-#endif
-#if !defined(LUTGEMM_DEV_ONLY_Q) || LUTGEMM_DEV_ONLY_Q == 7
         case 7: return launch_off<7>(has_offset, gsub, a, workgroups, th, stream);
-#endif
-#if !defined(LUTGEMM_DEV_ONLY_Q) || LUTGEMM_DEV_ONLY_Q == 8
         case 8: return launch_off<8>(has_offset, gsub, a, workgroups, th, stream);
-#endif
         default: return hipErrorInvalidValue;
     }
 }
