@@ -20,7 +20,11 @@
  *
  * Parity status of every exported function is "pinned": each one is checked in
  * tests/test_oracle.py against something it does not itself compute (numpy float16,
- * numpy unpackbits + dense matmul, closed forms, brute force on tiny inputs).
+ * numpy unpackbits + dense matmul, closed forms, brute force on tiny inputs); the order of
+ * the fp16 operations in orc_ref_kernel_fp16 is pinned in tests/test_oracle_ref_kernel.py by
+ * known answers worked out by hand from the reference source, where binary16 rounding makes
+ * every other order give a different number, and by a thread-by-thread transcription of the
+ * CUDA kernels in numpy.float16 that must agree bit for bit.
  *
  * Layout conventions (reference names in brackets):
  *   K [kSize]  reduction length, multiple of 32

@@ -212,8 +212,8 @@ def test_rtn_to_bcq_identity_exhaustive(oracle):
 @pytest.mark.parametrize("offset", [False, True])
 def test_ref_kernel_emulation_exact_when_nothing_rounds(oracle, offset):
     """With small integer activations and unit scales every fp16 operation is exact, so the
-    emulated kernel must reproduce the truth exactly.  (The rounding order on general data
-    cannot be checked without a CUDA device; it is reported, never used as a pass criterion.)"""
+    emulated kernel must reproduce the truth exactly.  (The order of its rounding steps is pinned
+    in test_oracle_ref_kernel.py.)"""
     rng = np.random.default_rng(10)
     K, N, q, g = 256, 8, 3, 128
     bW = rng.integers(0, 2 ** 32, size=(K // 32, q, N), dtype=np.uint32)
