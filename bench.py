@@ -107,6 +107,22 @@ def cpu_baseline(synth, cfg, x16, w, truth, slice_n=12288):
     }
 
 
+PARITY_FAILURES = []   # filled by parity_record; a non-empty list makes the run exit with status 1
+
+
+def parity_record(oracle, y16, truth, n_chk, label=""):
+    """Error statistics of an fp16 result against the float64 truth, and the verdict of the
+    path's tolerance (oracle.tolerance_violation); a violation is remembered for the exit status."""
+    mean_abs, max_abs, rel_l2 = oracle.error_stats(y16, truth)
+    bad = oracle.tolerance_violation(y16, truth)
+    if bad is not None:
+        PARITY_FAILURES.append("%s%s" % (label + ": " if label else "", bad))
+    return {"truth": "fp64 accumulation over fp16-rounded inputs (oracle)", "outputs_checked": n_chk,
+            "mean_abs": mean_abs, "max_abs": max_abs, "rel_l2": rel_l2,
+            "tolerance": "|y-y*| <= %g ulp_fp16(|y*|) + %g and rel L2 <= %g" % (oracle.ULPS, oracle.ABS_TOL, oracle.REL_L2_TOL),
+            "within_tolerance": bad is None, "violation": bad}
+
+
 class Point:
     """One weight shape on the device: R rotating copies, an autotuned plan, buffers."""
 
@@ -147,27 +163,59 @@ class Point:
                                   np.ascontiguousarray(self.w["alpha"].astype(np.float16)[:, :, :n_chk]),
                                   np.ascontiguousarray(z) if z is not None else None, self.x16)
         y = self.yd[0].cpu().numpy()[:, :n_chk]
-        mean_abs, max_abs, rel_l2 = oracle.error_stats(y, truth)
-        return {"truth": "fp64 accumulation over fp16-rounded inputs (oracle)", "outputs_checked": n_chk,
-                "mean_abs": mean_abs, "max_abs": max_abs, "rel_l2": rel_l2}, truth
+        return parity_record(oracle, y, truth, n_chk), truth
 
     def close(self):
         for wgt in self.weights:
             wgt.close()
 
 
+PREWARM_MS = 40.0   # the device reaches its sustained clocks only after some tens of ms under load
+BURSTS = 15         # the --steps burst is timed this many times back to back; the median is reported
+
+
+def prewarm(torch, launch, min_ms=PREWARM_MS):
+    """Keep the device busy with `launch` (a burst of the workload's own launches) for min_ms."""
+    t0 = time.perf_counter()
+    while (time.perf_counter() - t0) * 1e3 < min_ms:
+        launch()
+        launch()
+        torch.cuda.synchronize()
+
+
+def time_bursts(torch, stream, launches):
+    """Each callable in `launches` issues one burst; all bursts are issued back to back, each
+    bracketed by HIP events on the launch stream.  Returns the burst times in ms."""
+    ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in launches]
+    for (e0, e1), fn in zip(ev, launches):
+        e0.record(stream)
+        fn()
+        e1.record(stream)
+    torch.cuda.synchronize()
+    return [e0.elapsed_time(e1) for e0, e1 in ev]
+
+
+def median(v):
+    v = sorted(v)
+    n = len(v)
+    return v[n // 2] if n % 2 else 0.5 * (v[n // 2 - 1] + v[n // 2])
+
+
 def time_point(lutgemm, torch, stream, pt, steps, warmup):
+    """us per step, rotating copies and single copy: `warmup` untimed steps, then (whatever
+    `warmup` is) PREWARM_MS of launches so that the clocks are up, then BURSTS bursts of exactly
+    `steps` steps; the median burst counts.  The rotation over the weight copies continues from
+    burst to burst, so no burst finds its weights in the memory-side cache."""
     sh = stream.cuda_stream
-    warm = lutgemm.MatvecSequence(pt.items(max(1, warmup)))
-    timed = lutgemm.MatvecSequence(pt.items(steps))
+    lutgemm.MatvecSequence(pt.items(max(1, warmup))).launch(sh)
+    torch.cuda.synchronize()
+    seqs = [lutgemm.MatvecSequence(pt.items(steps, offset=b * steps)) for b in range(BURSTS)]
     hot = lutgemm.MatvecSequence(pt.items(steps, rotate=False))
-    warm.launch(sh)
-    torch.cuda.synchronize()
-    ms = event_time_ms(torch, lambda: timed.launch(sh), stream)
-    torch.cuda.synchronize()
-    ms_hot = event_time_ms(torch, lambda: hot.launch(sh), stream)
-    torch.cuda.synchronize()
-    return ms * 1e3 / steps, ms_hot * 1e3 / steps
+    prewarm(torch, lambda: seqs[0].launch(sh))
+    ms = time_bursts(torch, stream, [(lambda q=q: q.launch(sh)) for q in seqs])
+    ms_hot = time_bursts(torch, stream, [lambda: hot.launch(sh)] * BURSTS)
+    pt.burst_us = [t * 1e3 / steps for t in ms]
+    return median(ms) * 1e3 / steps, median(ms_hot) * 1e3 / steps
 
 
 def point_record(pt, us, us_hot):
@@ -208,26 +256,27 @@ def run_single(args, lutgemm, synth, torch, dev, stream, name):
                      {"weight_copies_rotated": pt.copies, "packed_weight_bytes": pt.b_w, "plan": pt.plan})
     line["ms_per_step"] = us / 1e3
     kernel = "lut_matvec_kernel<%d,%s,1>" % (q, "true" if pt.has_offset else "false")
+    traffic = CFG1_MEASURED_TRAFFIC_BYTES.get(pt.plan["k_splits"]) if name == "cfg1" else None
     line["roofline"] = {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                        "frac": achieved / HBM_PEAK_GBS,
-                        "traffic": CFG1_MEASURED_TRAFFIC_BYTES.get(pt.plan["k_splits"]) if name == "cfg1" else None,
-                        "kernel": kernel, "algorithmic_bytes_per_launch": pt.b_total, "avg_launch_us": us}
+                        "frac": achieved / HBM_PEAK_GBS, "traffic": traffic,
+                        "traffic_source": (
+                            "not measured in this run: rocprofv3 --pmc FETCH_SIZE x 2.000 + WRITE_SIZE x 1.000 per dispatch for "
+                            "this launch plan, from profiles/lut_matvec_kernel_cfg1.md" if traffic is not None else
+                            "no counter run on record for this workload and launch plan (profiles/)"),
+                        "kernel": kernel, "algorithmic_bytes_per_launch": pt.b_total, "avg_launch_us": us,
+                        "launch_us_bursts": pt.burst_us}
     line["hot_single_copy"] = {"us_per_matvec": us_hot, "weight_GBps": pt.b_w / (us_hot * 1e-6) / 1e9}
-    # the device's pure-read time for the same tiles, same grid, same rotation over the copies
-    # (warmed like the matvec: the device only reaches its sustained clocks under load)
-    lutgemm.read_probe([pt.weights[i % pt.copies] for i in range(max(1, args.warmup))], stream.cuda_stream)
-    torch.cuda.synchronize()
+    # the device's pure-read time for the same tiles, same grid, same rotation over the copies,
+    # timed like the matvec (clocks warmed, median of BURSTS bursts)
     reads = max(1, args.steps)
-    order = [pt.weights[i % pt.copies] for i in range(reads)]
-
-    def run_reads():
-        lutgemm.read_probe(order, stream.cuda_stream)
-    rms = event_time_ms(torch, run_reads, stream)
-    read_us = rms * 1e3 / reads
-    info = pt.weights[0].info()
-    tile_bytes = info.device_bytes - 8 * 2 * 32 * ((n + 31) // 32)  # packed tiles incl. padding, without the split-k words
+    orders = [[pt.weights[(b * reads + i) % pt.copies] for i in range(reads)] for b in range(BURSTS)]
+    prewarm(torch, lambda: lutgemm.read_probe(orders[0], stream.cuda_stream))
+    rms = time_bursts(torch, stream, [(lambda o=o: lutgemm.read_probe(o, stream.cuda_stream)) for o in orders])
+    read_us = median(rms) * 1e3 / reads
+    tile_bytes = sum(lutgemm.packed_sizes(k, n, q, k // g, pt.has_offset))  # packed tiles incl. padding
     line["pure_read_same_tiles"] = {"us": read_us, "bytes": tile_bytes, "GBps": tile_bytes / read_us / 1e3,
                                     "matvec_time_over_read_time": us / read_us}
+    line["roofline"]["read_floor_us"] = read_us
     if name == "cfg1":
         import numpy as np
         from oracle import oracle
@@ -252,10 +301,12 @@ def run_single(args, lutgemm, synth, torch, dev, stream, name):
         Wd = [torch.randn((n, k), dtype=torch.float16, device=dev) * 0.03 for _ in range(nd)]
         xv = pt.xd[0]
         outs = torch.empty((nd, n), dtype=torch.float16, device=dev)
-        for i in range(10):
-            torch.mv(Wd[i % nd], xv, out=outs[i % nd])
-        torch.cuda.synchronize()
         reps = 50
+
+        def warm_dense():
+            for i in range(10):
+                torch.mv(Wd[i % nd], xv, out=outs[i % nd])
+        prewarm(torch, warm_dense)
 
         def run_dense():
             for i in range(reps):
@@ -343,11 +394,11 @@ def run_cfg4(args, lutgemm, synth, torch, dev, stream):
                 out.extend(pts[nm].items(1, offset=s))
         return out
 
-    warm = lutgemm.MatvecSequence(chain_items(max(1, args.warmup)))
-    timed = lutgemm.MatvecSequence(chain_items(args.steps))
-    warm.launch(sh)
+    lutgemm.MatvecSequence(chain_items(max(1, args.warmup))).launch(sh)
     torch.cuda.synchronize()
-    ms = event_time_ms(torch, lambda: timed.launch(sh), stream)
+    timed = lutgemm.MatvecSequence(chain_items(args.steps))
+    prewarm(torch, lambda: timed.launch(sh))
+    ms = median(time_bursts(torch, stream, [lambda: timed.launch(sh)] * 7))
     chain_us = ms * 1e3 / args.steps
     graph = None
     if args.graph:
@@ -433,8 +484,10 @@ def run_dequant(args, lutgemm, synth, torch, dev, stream):
         dense = oracle.dense_weight_f64(np.ascontiguousarray(w["bW"][:, :, :256]),
                                         np.ascontiguousarray(w["alpha"].astype(np.float16)[:, :, :256]),
                                         np.ascontiguousarray(z) if z is not None else None)
-        rec["parity"] = {"outputs_checked": 256,
-                         "within_half_ulp_fp16": bool(np.all(np.abs(got - dense) <= 2.0 ** -11 * np.abs(dense) + 2.0 ** -24))}
+        exact = bool(np.all(np.abs(got - dense) <= 2.0 ** -11 * np.abs(dense) + 2.0 ** -24))
+        rec["parity"] = {"outputs_checked": 256, "within_half_ulp_fp16": exact}
+        if not exact:
+            PARITY_FAILURES.append("dequantize %s: more than half an fp16 ulp from the dense weight" % name)
         shapes.append(rec)
         W.close()
         del outs
@@ -493,7 +546,9 @@ def main():
         line = run_dequant(args, lutgemm, synth, torch, dev, stream)
     else:
         line = run_single(args, lutgemm, synth, torch, dev, stream, args.config)
-    print(json.dumps(line))
+    print(json.dumps(line), flush=True)
+    if PARITY_FAILURES:
+        sys.exit("bench.py: result outside the tolerance of the path: " + "; ".join(PARITY_FAILURES))
 
 
 if __name__ == "__main__":

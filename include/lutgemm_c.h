@@ -39,7 +39,7 @@ typedef enum lutgemm_status {
 } lutgemm_status;
 
 /* Opaque packed weight: device-resident sign tiles, scales and offsets plus the launch plan
- * and the split-k accumulators (one 64-bit word per output).  Stands in for class lutGEMM::nQWeight_fp16
+ * and the split-k accumulators (64-bit words, two per output and launching stream).  Stands in for class lutGEMM::nQWeight_fp16
  * (lutGEMM/include/nQWeight_fp16.h:27-52). */
 typedef struct lutgemm_weight lutgemm_weight;
 
@@ -88,11 +88,15 @@ int lutgemm_weight_info(const lutgemm_weight *w, lutgemm_weight_info_t *info);
  * kernel::nqmv (mv_fp16.hpp:121) or kernel::nqmv_bias (mv_fp16_bias.hpp:143); here every
  * 1 <= m <= LUTGEMM_MAX_BATCH stays on the table-lookup kernels: rows go through the weight two
  * per pass (one for a last odd row), every row bit-identical to its own one-row call.
- * Calls that overlap in time on the same handle race on its split-k accumulators.
- * Finite inputs are assumed: with more than one k-split the partial sums are added as fixed-point
- * integers (2^-24 resolution, saturating at about +-8.4e6, far beyond binary16's range), so an
- * infinite partial sum still yields an infinity of that sign, but a NaN one yields an infinity
- * instead of a NaN. */
+ * Launches on one stream run one after the other and share the handle's split-k accumulators;
+ * every further stream that launches on the handle gets accumulators of its own (eight streams
+ * per handle, LUTGEMM_ERR_UNSUPPORTED beyond; lutgemm_weight_reset_workspace releases them), so
+ * launches on different streams may overlap in time.  Launches from different host threads on the
+ * SAME stream must be serialised by the caller, as for any stream.
+ * Non-finite values follow IEEE arithmetic whatever the launch plan: a NaN activation gives NaN
+ * outputs, infinite partial sums give an infinity of their sign, or NaN if both signs occur.  With
+ * more than one k-split the partial sums are added as fixed-point integers (2^-24 resolution);
+ * a finite partial sum beyond +-4.1e6 (64 times binary16's range) counts as an infinity. */
 #define LUTGEMM_MAX_BATCH 4096
 int lutgemm_matvec(const lutgemm_weight *w, const void *x, void *y, int m, void *stream);
 
@@ -100,8 +104,8 @@ int lutgemm_matvec(const lutgemm_weight *w, const void *x, void *y, int m, void 
  * Replaces lutGEMM::matmul(void* output, nQWeight_fp16&, void* input, int n, int algo)
  * (lutGEMM/include/kernels.h:26, lutGEMM/src/kernels.cu:56-63).  For m == 1 it is the same
  * operation as lutgemm_matvec.  For m > 1 the columns are first gathered into a staging buffer
- * owned by the handle; the buffer is allocated (and the stream synchronised) the first time a
- * given m is exceeded. */
+ * owned by the handle (one per launching stream).  Up to m = 8 nothing is allocated; a larger m
+ * grows the buffer the first time it occurs (device synchronisation, free and allocation). */
 int lutgemm_matvec_cols(const lutgemm_weight *w, const void *x, void *y, int m, void *stream);
 
 /* `count` independent matvecs issued back to back on one stream with a single call (for a
@@ -111,6 +115,14 @@ int lutgemm_matvec_cols(const lutgemm_weight *w, const void *x, void *y, int m, 
  * (tests/opt/fp16/int3_col_wise_matmul_fp16.cu:120-133).  Stops at the first failing entry. */
 int lutgemm_matvec_many(const lutgemm_weight *const *ws, const void *const *xs, void *const *ys,
                         const int *ms, int count, void *stream);
+
+/* Put every split-k accumulator of the handle back to zero and forget which streams have
+ * launched on it (synchronises the device, then runs a fill kernel on `stream` and waits for it).
+ * Only needed after a launch was aborted half way (a failed launch in the middle of a batched call,
+ * a device fault): completed launches always leave their accumulators at zero.  No counterpart in
+ * the reference, which clears its output with cudaMemset before every call
+ * (lutGEMM/src/kernels.cu:66). */
+int lutgemm_weight_reset_workspace(lutgemm_weight *w, void *stream);
 
 /* Dense fp16 weight on the device, W[k][n] (transposed == 0) or W[n][k] (transposed != 0),
  * offset included.  d_fW is a device pointer to k*n halves.  Asynchronous on `stream`.
@@ -152,7 +164,8 @@ int lutgemm_weight_set_plan(lutgemm_weight *w, int waves_per_group, int k_splits
 
 /* Measure the most promising launch plans on the device (a few launches each, on `stream`, with
  * scratch activations of its own) and keep the fastest, separately for launches with one
- * activation row and for two-row passes.  Optional: the automatic plan is chosen
+ * activation row and for two-row passes (which keep the k-split of the one-row plan, so that
+ * rows stay bit-identical to their own one-row launches).  Optional: the automatic plan is chosen
  * from a model, this replaces it by a measurement.  The measurement streams the weight from
  * HBM as a decoder does: it rotates over temporary device copies of the packed weight (about
  * 1 GiB in total, at most 64 copies) so that no launch finds its weight in the memory-side
@@ -205,8 +218,7 @@ int lutgemm_weight_save(const lutgemm_weight *w, const char *path);
 int lutgemm_weight_load(const char *path, lutgemm_weight **out);
 
 /* A second, independent handle with its own device copy of the packed weight and its own
- * workspace (device-to-device copy, no packing), with the same launch plan.  Handles must not
- * be shared by launches that overlap in time; clones can be. */
+ * workspace (device-to-device copy, no packing), with the same launch plan. */
 int lutgemm_weight_clone(const lutgemm_weight *w, lutgemm_weight **out);
 
 /* float -> binary16 bit patterns, round to nearest even: the conversion applied to alpha and

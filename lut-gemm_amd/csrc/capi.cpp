@@ -11,6 +11,7 @@
 #include <cstdint>
 #include <cstdio>
 #include <cstring>
+#include <mutex>
 #include <new>
 #include <vector>
 
@@ -41,7 +42,10 @@ int hip_fail(hipError_t e, const char *what)
 
 constexpr int kMaxWaves = 12;  // the kernel is compiled for at most 768 threads per workgroup
 constexpr int kBuildRounds = 8;  // table parts per k-block (kernels.hip: kBuildParts)
-constexpr int kMaxSplits = 128;  // the split-k arrival count has 8 bits and the sum 2^56 / 2^48 addends
+constexpr int kMaxSplits = 128;  // the split-k arrival count has 8 bits, the sum room for 128 addends
+constexpr int kStreamSlots = 8;  // sets of split-k words per handle: one per stream that launches on it
+constexpr int kRowsPerPass = 2;  // activation rows a launch can take (rows of split-k words per slot)
+constexpr int kStagedColumns = 8;  // column-batched calls up to this m never allocate
 
 struct Plan {
     int waves;             // wavefronts (= output batches) per workgroup
@@ -58,12 +62,20 @@ struct lutgemm_weight {
     int compute_units;
     uint8_t *d_signs;
     uint16_t *d_scales;
-    unsigned long long *d_accum;  // split-k accumulators, one 64-bit word per (padded) output
+    // Split-k accumulators: kStreamSlots sets of kRowsPerPass x (padded outputs) 64-bit words.
+    // Launches on one stream run one after the other and share a set; every other stream that
+    // launches on this handle gets a set of its own, so launches that overlap on different
+    // streams never touch the same words.
+    unsigned long long *d_accum;
     size_t accum_bytes;
-    void *d_xrows;                // staging for column-batched activations, grown on demand
-    size_t xrows_bytes;
+    size_t slot_words;
+    std::mutex slot_mutex;
+    void *slot_stream[kStreamSlots];
+    int slots_used;
+    void *d_xrows;                // staging for column-batched activations: per stream set
+    int xrows_cols;               //   xrows_cols rows of k halves; grown on demand beyond that
     Plan plan;                    // launches with one activation row
-    Plan plan2;                   // passes over two activation rows (m >= 2)
+    Plan plan2;                   // passes over two activation rows (m >= 2): same k-split as plan
 };
 
 namespace {
@@ -131,11 +143,36 @@ int check_device(const lutgemm_weight *w)
 int alloc_workspace(lutgemm_weight *w)
 {
     if (w->d_accum) return LUTGEMM_OK;  // size depends on the shape only
-    w->accum_bytes = 2 * (size_t)w->shape.nb * kBatch * sizeof(unsigned long long);  // two rows per pass
+    w->slot_words = (size_t)kRowsPerPass * w->shape.nb * kBatch;
+    w->accum_bytes = (size_t)kStreamSlots * w->slot_words * sizeof(unsigned long long);
     hipError_t e = hipMalloc((void **)&w->d_accum, w->accum_bytes);
     if (e != hipSuccess) return hip_fail(e, "hipMalloc(split-k accumulators)");
     e = hipMemset(w->d_accum, 0, w->accum_bytes);
     if (e != hipSuccess) return hip_fail(e, "hipMemset(split-k accumulators)");
+    e = hipMalloc(&w->d_xrows, (size_t)kStreamSlots * kStagedColumns * w->shape.k * sizeof(uint16_t));
+    if (e != hipSuccess) return hip_fail(e, "hipMalloc(column staging)");
+    w->xrows_cols = kStagedColumns;
+    return LUTGEMM_OK;
+}
+
+// The split-k words launches on `stream` use.  The first launch of a stream on this handle claims
+// a set; kStreamSlots streams can use one handle at a time (clones have sets of their own).
+int stream_words(lutgemm_weight *w, void *stream, unsigned long long **words, int *slot)
+{
+    std::lock_guard<std::mutex> lock(w->slot_mutex);
+    for (int i = 0; i < w->slots_used; i++)
+        if (w->slot_stream[i] == stream) {
+            *words = w->d_accum + (size_t)i * w->slot_words;
+            *slot = i;
+            return LUTGEMM_OK;
+        }
+    if (w->slots_used == kStreamSlots)
+        return fail(LUTGEMM_ERR_UNSUPPORTED,
+                    "more than %d streams have launched on this handle; use lutgemm_weight_clone for "
+                    "further streams or lutgemm_weight_reset_workspace to release the sets", kStreamSlots);
+    w->slot_stream[w->slots_used] = stream;
+    *words = w->d_accum + (size_t)w->slots_used * w->slot_words;
+    *slot = w->slots_used++;
     return LUTGEMM_OK;
 }
 
@@ -315,10 +352,10 @@ int run_matvec(const lutgemm_weight *w, const void *x, void *y, int m, void *str
         return fail(LUTGEMM_ERR_BAD_SHAPE, "m=%d outside 1..%d", m, LUTGEMM_MAX_BATCH);
     if (int st_dev = check_device(w)) return st_dev;
     const Shape &s = w->shape;
+    lutgemm_weight *mw = const_cast<lutgemm_weight *>(w);
     lutgemm_kernels::MatvecArgs a{};
     a.signs = w->d_signs;
     a.scales = w->d_scales;
-    a.accum = w->d_accum;
     a.k = s.k;
     a.n = s.n;
     a.ts = s.ts;
@@ -328,23 +365,28 @@ int run_matvec(const lutgemm_weight *w, const void *x, void *y, int m, void *str
     if (((uintptr_t)x & 15u) != 0)  // rows of x are k fp16 apart and k is a multiple of 32
         return fail(LUTGEMM_ERR_BAD_SHAPE, "x must be 16-byte aligned");
     hipStream_t st = static_cast<hipStream_t>(stream);
+    int slot = 0;
+    if (int st_ws = stream_words(mw, stream, &a.accum, &slot)) {
+        return st_ws;
+    }
     if (cols && m > 1) {
         // gather the m columns into contiguous rows first (the kernel reads 16 bytes per lane)
-        lutgemm_weight *mw = const_cast<lutgemm_weight *>(w);
-        const size_t need = (size_t)m * s.k * sizeof(uint16_t);
-        if (mw->xrows_bytes < need) {
-            hipError_t e = hipStreamSynchronize(st);  // an earlier launch may still read the old buffer
-            if (e != hipSuccess) return hip_fail(e, "hipStreamSynchronize");
+        if (m > mw->xrows_cols) {
+            // an earlier launch on any stream may still read the old buffer
+            std::lock_guard<std::mutex> lock(mw->slot_mutex);
+            hipError_t e = hipDeviceSynchronize();
+            if (e != hipSuccess) return hip_fail(e, "hipDeviceSynchronize");
             if (mw->d_xrows) (void)hipFree(mw->d_xrows);
             mw->d_xrows = nullptr;
-            mw->xrows_bytes = 0;
-            e = hipMalloc(&mw->d_xrows, need);
+            mw->xrows_cols = 0;
+            e = hipMalloc(&mw->d_xrows, (size_t)kStreamSlots * m * s.k * sizeof(uint16_t));
             if (e != hipSuccess) return hip_fail(e, "hipMalloc(column staging)");
-            mw->xrows_bytes = need;
+            mw->xrows_cols = m;
         }
-        hipError_t e = lutgemm_kernels::launch_gather_columns(x, mw->d_xrows, s.k, m, st);
+        uint16_t *rows = static_cast<uint16_t *>(mw->d_xrows) + (size_t)slot * mw->xrows_cols * s.k;
+        hipError_t e = lutgemm_kernels::launch_gather_columns(x, rows, s.k, m, st);
         if (e != hipSuccess) return hip_fail(e, "launch gather_columns_kernel");
-        xh = static_cast<const uint16_t *>(mw->d_xrows);
+        xh = rows;
     }
     // two activation rows per pass over the weight, a last single row if m is odd
     a.x_row_stride = s.k;
@@ -504,6 +546,22 @@ int lutgemm_weight_info(const lutgemm_weight *w, lutgemm_weight_info_t *info)
 int lutgemm_matvec(const lutgemm_weight *w, const void *x, void *y, int m, void *stream)
 {
     return run_matvec(w, x, y, m, stream, false);
+}
+
+int lutgemm_weight_reset_workspace(lutgemm_weight *w, void *stream)
+{
+    if (!w) return fail(LUTGEMM_ERR_NULL_POINTER, "null argument to weight_reset_workspace");
+    if (int st_dev = check_device(w)) return st_dev;
+    std::lock_guard<std::mutex> lock(w->slot_mutex);
+    hipError_t e = hipDeviceSynchronize();  // no launch may still be using the words
+    if (e != hipSuccess) return hip_fail(e, "hipDeviceSynchronize");
+    e = lutgemm_kernels::launch_fill_zero(w->d_accum, w->accum_bytes / sizeof(unsigned long long),
+                                          static_cast<hipStream_t>(stream));
+    if (e != hipSuccess) return hip_fail(e, "launch fill_zero_kernel");
+    e = hipStreamSynchronize(static_cast<hipStream_t>(stream));
+    if (e != hipSuccess) return hip_fail(e, "hipStreamSynchronize");
+    w->slots_used = 0;
+    return LUTGEMM_OK;
 }
 
 int lutgemm_matvec_cols(const lutgemm_weight *w, const void *x, void *y, int m, void *stream)
@@ -731,7 +789,18 @@ int lutgemm_weight_autotune(lutgemm_weight *w, void *stream)
     for (int rows = 1; rows <= 2; rows++) {
         struct Timed { float ms; Plan p; };
         std::vector<Timed> timed;
-        for (size_t i = 0; status == LUTGEMM_OK && i < cands.size(); i++) timed.push_back(Timed{1e30f, cands[i].p});
+        if (rows == 1) {
+            for (size_t i = 0; status == LUTGEMM_OK && i < cands.size(); i++) timed.push_back(Timed{1e30f, cands[i].p});
+        } else {
+            // Rows of a two-row pass must come out bit for bit as their own one-row launch does:
+            // same k-split (same partial sums); only the wavefronts per workgroup may differ.
+            for (int waves = 1; waves <= kMaxWaves; waves++) {
+                Plan p = chosen[0];
+                p.waves = waves;
+                p.ntiles = div_up(s.nb, waves);
+                timed.push_back(Timed{1e30f, p});
+            }
+        }
         for (int sweep = 0; sweep < 2; sweep++)
             for (size_t i = 0; status == LUTGEMM_OK && i < timed.size(); i++) {
                 float ms = 0.f;

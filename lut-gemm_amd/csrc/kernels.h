@@ -13,7 +13,7 @@ struct MatvecArgs {
     const uint16_t *scales; // scale tiles (layout.h)
     const void *x;          // fp16 activations, contiguous, 16-byte aligned
     void *y;                // fp16 outputs, element j at y[j * y_stride]
-    unsigned long long *accum;  // [2][nb*32] split-k accumulators (count | fixed-point sum), zero
+    unsigned long long *accum;  // [2][nb*32] split-k accumulators (count | flags | fixed-point sum), zero
                                 // between launches; used when k_splits > 1
     int k, n;
     int ts, nb;             // k-blocks, output batches
@@ -38,6 +38,9 @@ struct DequantArgs {
 // workgroups = ntiles * k_splits, `waves` wavefronts of 64 lanes per workgroup.
 hipError_t launch_matvec(int q, int has_offset, int gsub, const MatvecArgs &a, int workgroups,
                          int waves, hipStream_t stream);
+
+// words[0..count) = 0 (a fill kernel rather than a memset node, so that it can be captured)
+hipError_t launch_fill_zero(unsigned long long *words, size_t count, hipStream_t stream);
 
 // fp16 [k][m] -> [m][k]
 hipError_t launch_gather_columns(const void *cols, void *rows, int k, int m, hipStream_t stream);

@@ -483,12 +483,19 @@ __device__ __forceinline__ float reduce_across_lanes(float (&acc)[kBatch], int l
 // Lane pair (2j, 2j+1) of a wavefront holds the k-range total of output `out`; the even lane
 // delivers it.  With one k-split it is the result.  Otherwise: one 64-bit atomic add per output,
 // no barrier, no second pass.  The word holds an arrival count in its top 8 bits and the running
-// sum below it, as a biased fixed-point integer (2^-24 units, bias 2^47 per addend so every
-// addend is positive and the sum never carries into the count).  Integer addition is
-// associative, so the total does not depend on the order in which the workgroups arrive: the
-// result is deterministic.  The workgroup whose add returns count == k_splits-1 is the last one
-// for that output: it holds the complete sum, writes y and puts the word back to zero for the
-// next launch.
+// sum below it, as a biased fixed-point integer (2^-24 units, bias 2^46 per addend so every
+// addend is positive; at most 128 addends below 2^47 keep the sum below 2^54 and out of the
+// flags and the count).  Integer addition is associative, so the total does not depend on the
+// order in which the workgroups arrive: the result is deterministic.  The workgroup whose add
+// returns count == k_splits-1 is the last one for that output: it holds the complete sum, writes
+// y and puts the word back to zero for the next launch.
+// A partial sum that is not finite cannot be expressed in fixed point.  Its workgroup first sets
+// a flag in the same word (bit 54: +infinity seen, bit 55: -infinity seen, both: NaN) and then
+// adds a zero contribution; the finishing workgroup turns the flags into the value IEEE
+// arithmetic gives the sum: +-infinity, or NaN for a NaN or for infinities of both signs.  The
+// flag store and the add are atomics of one thread on one address, so they take effect in
+// program order.
+constexpr unsigned long long kPosInfFlag = 1ull << 54, kNegInfFlag = 1ull << 55;
 __device__ __forceinline__ void finish_output(float total, bool active, int out, int lane, __half *y,
                                               unsigned long long *accum, const MatvecArgs &a)
 {
@@ -497,16 +504,28 @@ __device__ __forceinline__ void finish_output(float total, bool active, int out,
         y[(size_t)out * a.y_stride] = __float2half_rn(total);
         return;
     }
-    const float scaled = fminf(fmaxf(total * 16777216.f, -1.4e14f), 1.4e14f);  // |v| < 2^47
-    const unsigned long long addend =
-        (unsigned long long)(__float2ll_rn(scaled) + (1ll << 47)) + (1ull << 56);
     unsigned long long *word = accum + out;
+    float scaled = total * 16777216.f;
+    if (!(fabsf(scaled) < 7.0e13f)) {  // beyond 2^46 in fixed point, infinite or NaN
+        const unsigned long long flags =
+            total != total ? (kPosInfFlag | kNegInfFlag) : total > 0.f ? kPosInfFlag : kNegInfFlag;
+        __hip_atomic_fetch_or(word, flags, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        scaled = 0.f;
+    }
+    const unsigned long long addend =
+        (unsigned long long)(__float2ll_rn(scaled) + (1ll << 46)) + (1ull << 56);
     const unsigned long long old =
         __hip_atomic_fetch_add(word, addend, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     if ((old >> 56) == (unsigned long long)(a.k_splits - 1)) {
-        const unsigned long long sum = (old + addend) & ((1ull << 56) - 1);
-        const long long value = (long long)sum - (long long)a.k_splits * (1ll << 47);
-        y[(size_t)out * a.y_stride] = __float2half_rn(__ll2float_rn(value) * (1.f / 16777216.f));
+        const unsigned long long all = old + addend;
+        const long long value = (long long)(all & (kPosInfFlag - 1)) - (long long)a.k_splits * (1ll << 46);
+        float result = __ll2float_rn(value) * (1.f / 16777216.f);
+        const unsigned long long flags = all & (kPosInfFlag | kNegInfFlag);
+        if (flags)
+            result = flags == kPosInfFlag   ? __builtin_inff()
+                     : flags == kNegInfFlag ? -__builtin_inff()
+                                            : __builtin_nanf("");
+        y[(size_t)out * a.y_stride] = __float2half_rn(result);
         __hip_atomic_store(word, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
 }
@@ -769,6 +788,12 @@ __global__ __launch_bounds__(256) void gather_columns_kernel(const uint16_t *col
     rows[idx] = cols[(size_t)i * m + r];
 }
 
+__global__ __launch_bounds__(256) void fill_zero_kernel(unsigned long long *words, size_t count)
+{
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < count; i += (size_t)gridDim.x * blockDim.x)
+        words[i] = 0ull;
+}
+
 template <int Q, bool OFF, int GSUB>
 hipError_t launch_one(const MatvecArgs &a, int workgroups, int threads, hipStream_t stream)
 {
@@ -830,6 +855,15 @@ hipError_t launch_matvec(int q, int has_offset, int gsub, const MatvecArgs &a, i
         case 8: return launch_off<8>(has_offset, gsub, a, workgroups, th, stream);
         default: return hipErrorInvalidValue;
     }
+}
+
+hipError_t launch_fill_zero(unsigned long long *words, size_t count, hipStream_t stream)
+{
+    if (count == 0) return hipSuccess;
+    const size_t blocks = (count + 255) / 256;
+    hipLaunchKernelGGL(fill_zero_kernel, dim3((unsigned)(blocks < 1024 ? blocks : 1024)), dim3(256), 0, stream, words,
+                       count);
+    return hipGetLastError();
 }
 
 hipError_t launch_gather_columns(const void *cols, void *rows, int k, int m, hipStream_t stream)

@@ -31,6 +31,7 @@ EXPORTED = [
     "lutgemm_pack_host", "lutgemm_unpack_host", "lutgemm_float_to_half", "lutgemm_last_error",
     "lutgemm_status_string", "lutgemm_version", "lutgemm_pack_file", "lutgemm_unpack_file", "lutgemm_weight_save",
     "lutgemm_weight_load", "lutgemm_weight_clone", "lutgemm_read_probe", "lutgemm_dense_gemv_f16",
+    "lutgemm_weight_reset_workspace",
 ]
 
 
@@ -90,6 +91,7 @@ def load():
     L.lutgemm_read_probe.argtypes = [vp, i, vp]
     L.lutgemm_dense_gemv_f16.argtypes = [vp, vp, vp, i, i, vp]
     L.lutgemm_weight_set_plan.argtypes = [vp, i, i]
+    L.lutgemm_weight_reset_workspace.argtypes = [vp, vp]
     L.lutgemm_weight_autotune.argtypes = [vp, vp]
     L.lutgemm_weight_device_ptrs.argtypes = [vp, pp, pp, pp]
     L.lutgemm_packed_sizes.argtypes = [i, i, i, i, i, psz, psz]
@@ -254,6 +256,11 @@ class BCQWeight:
         """Measure candidate launch plans on the device and keep the fastest; returns the plan."""
         _check(load().lutgemm_weight_autotune(self._h, stream or None))
         return self.plan()
+
+    def reset_workspace(self, stream=0):
+        """Zero the split-k accumulators and release the per-stream sets (only needed after an
+        aborted launch)."""
+        _check(load().lutgemm_weight_reset_workspace(self._h, stream or None))
 
     def weight_bytes(self):
         """Algorithmic packed-weight bytes: signs + scales + offsets (unpadded)."""

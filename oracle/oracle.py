@@ -220,3 +220,39 @@ def error_stats(y_h, truth):
     out = np.zeros(3, np.float64)
     lib().orc_error_stats(_p(y_h), _p(truth), y_h.size, _p(out))
     return tuple(out)
+
+
+# Tolerance of the path (fp16 in/out, fp32 accumulation, one final rounding), against the
+# double-precision truth over the fp16-rounded inputs:
+#   per element  |y - y*| <= 2 ulp_fp16(|y*|) + 1e-3      and      ||y - y*||2 / ||y*||2 <= 1e-3
+ULPS = 2.0
+ABS_TOL = 1e-3
+REL_L2_TOL = 1e-3
+
+
+def ulp_fp16(v):
+    a = np.abs(np.asarray(v, np.float64))
+    e = np.floor(np.log2(np.maximum(a, 2.0 ** -14)))
+    return 2.0 ** (e - 10)
+
+
+def tolerance_violation(y16, truth):
+    """None if the fp16 result is within the tolerance above of the float64 truth, else a
+    description of the worst violation."""
+    y = np.asarray(y16, np.float16).astype(np.float64).reshape(-1)
+    t = np.asarray(truth, np.float64).reshape(-1)
+    if y.shape != t.shape:
+        return "shape mismatch: %r against %r" % (y.shape, t.shape)
+    if not np.all(np.isfinite(y)):
+        return "%d non-finite outputs" % int((~np.isfinite(y)).sum())
+    err = np.abs(y - t)
+    bound = ULPS * ulp_fp16(t) + ABS_TOL
+    if not np.all(err <= bound):
+        worst = int(np.argmax(err - bound))
+        return "element %d: got %r want %r err %g bound %g" % (worst, y[worst], t[worst], err[worst], bound[worst])
+    den = np.linalg.norm(t)
+    if den > 0:
+        rel = np.linalg.norm(y - t) / den
+        if rel > REL_L2_TOL:
+            return "relative L2 error %g above %g" % (rel, REL_L2_TOL)
+    return None

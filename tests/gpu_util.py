@@ -2,33 +2,14 @@
 tolerance of the path, and a runner that calls the product through its C ABI binding."""
 import numpy as np
 
-# Tolerance of the path (fp16 in/out, fp32 accumulation, one final rounding), against the
-# double-precision truth over the fp16-rounded inputs:
+# The tolerance of the path is stated once, next to the oracle (oracle/oracle.py):
 #   per element  |y - y*| <= 2 ulp_fp16(|y*|) + 1e-3      and      ||y - y*||2 / ||y*||2 <= 1e-3
-ULPS = 2.0
-ABS_TOL = 1e-3
-REL_L2_TOL = 1e-3
-
-
-def ulp_fp16(v):
-    a = np.abs(np.asarray(v, np.float64))
-    e = np.floor(np.log2(np.maximum(a, 2.0 ** -14)))
-    return 2.0 ** (e - 10)
+from oracle.oracle import ABS_TOL, REL_L2_TOL, ULPS, tolerance_violation, ulp_fp16  # noqa: F401
 
 
 def assert_within_tolerance(y16, truth, what=""):
-    y = np.asarray(y16, np.float16).astype(np.float64).reshape(-1)
-    t = np.asarray(truth, np.float64).reshape(-1)
-    assert np.all(np.isfinite(y)), what
-    err = np.abs(y - t)
-    bound = ULPS * ulp_fp16(t) + ABS_TOL
-    worst = int(np.argmax(err - bound))
-    assert np.all(err <= bound), "%s: element %d: got %r want %r err %g bound %g" % (
-        what, worst, y[worst], t[worst], err[worst], bound[worst])
-    den = np.linalg.norm(t)
-    if den > 0:
-        rel = np.linalg.norm(y - t) / den
-        assert rel <= REL_L2_TOL, "%s: relative L2 error %g" % (what, rel)
+    bad = tolerance_violation(y16, truth)
+    assert bad is None, "%s: %s" % (what, bad)
 
 
 def run_matvec(lg, weight, x16, device, cols=False):

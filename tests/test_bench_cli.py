@@ -20,3 +20,27 @@ def test_options():
     for opt in ("--gpus", "--steps", "--warmup", "--config", "--m", "--graph", "--plan", "--no-cpu", "--no-dense",
                 "--copy-calibration"):
         assert opt in r.stdout
+
+
+def test_parity_outside_the_tolerance_sets_the_exit_status(oracle):
+    """bench.py is a checker: a result outside the tolerance of the path is recorded and makes
+    the run exit with a non-zero status (here: a scale wrong by 1 %)."""
+    import importlib.util
+
+    import numpy as np
+    spec = importlib.util.spec_from_file_location("bench_under_test", BENCH)
+    bench = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(bench)
+    rng = np.random.default_rng(5)
+    K, N, q, g = 1024, 64, 3, 128
+    bW = rng.integers(0, 2 ** 32, size=(K // 32, q, N), dtype=np.uint32)
+    alpha = np.abs(rng.normal(0, 0.02, size=(K // g, q, N))).astype(np.float16)
+    x = rng.normal(0, 1, size=(1, K)).astype(np.float16)
+    truth = oracle.matvec_f64(bW, alpha, None, x)
+    good = truth.astype(np.float16)
+    rec = bench.parity_record(oracle, good, truth, N)
+    assert rec["within_tolerance"] and rec["violation"] is None and bench.PARITY_FAILURES == []
+    wrong = oracle.matvec_f64(bW, (alpha.astype(np.float32) * 1.01).astype(np.float16), None, x).astype(np.float16)
+    rec = bench.parity_record(oracle, wrong, truth, N, label="scaled")
+    assert not rec["within_tolerance"] and rec["violation"]
+    assert len(bench.PARITY_FAILURES) == 1 and bench.PARITY_FAILURES[0].startswith("scaled: ")
