@@ -100,6 +100,19 @@ int lutgemm_weight_info(const lutgemm_weight *w, lutgemm_weight_info_t *info);
 #define LUTGEMM_MAX_BATCH 4096
 int lutgemm_matvec(const lutgemm_weight *w, const void *x, void *y, int m, void *stream);
 
+/* lutgemm_matvec without any allocation, for callers that cannot allocate: code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc.  It has no counterpart in the
+ * reference.  Same arguments, same kernels and bit-identical results; the only difference is where
+ * the split-k accumulators live: not in the handle's allocation but in a static device array of
+ * the library (1 MiB on every device the library runs on, held until the process ends), whose
+ * address is looked up once per device.  Limit: n <= 65,536 outputs (LUTGEMM_ERR_UNSUPPORTED
+ * beyond).  The call performs no hipMalloc / hipFree and calls no allocating library routine.  All
+ * calls on one device share that device's array, whatever the handle or stream: calls that overlap
+ * in time on one device race on it (issue them on one stream, or use lutgemm_matvec, which keeps
+ * accumulators per handle and stream).  Completed launches leave the array at zero; after a launch
+ * that failed in the middle of a batched call the next call clears it with a fill kernel first. */
+int lutgemm_matvec_static(const lutgemm_weight *w, const void *x, void *y, int m, void *stream);
+
 /* Column-batched form: x is [k][m] and y is [n][m] (m vectors stored as columns).
  * Replaces lutGEMM::matmul(void* output, nQWeight_fp16&, void* input, int n, int algo)
  * (lutGEMM/include/kernels.h:26, lutGEMM/src/kernels.cu:56-63).  For m == 1 it is the same

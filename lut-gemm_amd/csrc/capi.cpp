@@ -176,6 +176,10 @@ int stream_words(lutgemm_weight *w, void *stream, unsigned long long **words, in
     return LUTGEMM_OK;
 }
 
+// The allocation-free entry point marks a device whose static split-k words a failed call may
+// have left non-zero; the next call on that device clears them first.
+bool g_static_dirty[lutgemm_kernels::kMaxDevices];
+
 // New handle for shape s on the current device from tiles already in the device layout
 // (host or device memory, `kind` says which).
 int create_from_tiles(const Shape &s, const void *signs, const void *scales, hipMemcpyKind kind,
@@ -345,7 +349,9 @@ int read_file(const char *path, Shape *s, std::vector<uint8_t> *signs, std::vect
     return st;
 }
 
-int run_matvec(const lutgemm_weight *w, const void *x, void *y, int m, void *stream, bool cols)
+// `static_ws`: take the split-k words from the static device array instead of the handle's
+// per-stream sets (rows form only; nothing on this route allocates).
+int run_matvec(const lutgemm_weight *w, const void *x, void *y, int m, void *stream, bool cols, bool static_ws)
 {
     if (!w || !x || !y) return fail(LUTGEMM_ERR_NULL_POINTER, "null argument to matvec");
     if (m < 1 || m > LUTGEMM_MAX_BATCH)
@@ -366,7 +372,20 @@ int run_matvec(const lutgemm_weight *w, const void *x, void *y, int m, void *str
         return fail(LUTGEMM_ERR_BAD_SHAPE, "x must be 16-byte aligned");
     hipStream_t st = static_cast<hipStream_t>(stream);
     int slot = 0;
-    if (int st_ws = stream_words(mw, stream, &a.accum, &slot)) {
+    if (static_ws) {
+        const size_t words = lutgemm_kernels::kStaticSplitKWords;
+        if ((size_t)kRowsPerPass * s.nb * kBatch > words)
+            return fail(LUTGEMM_ERR_UNSUPPORTED,
+                        "n=%d is beyond what the static workspace holds (%zu outputs per activation row)", s.n,
+                        words / kRowsPerPass);
+        hipError_t es = lutgemm_kernels::static_split_k_words(w->device, &a.accum);
+        if (es != hipSuccess) return hip_fail(es, "hipGetSymbolAddress(static split-k words)");
+        if (g_static_dirty[w->device]) {  // a launch failed half way through a call: start from zero again
+            hipError_t e = lutgemm_kernels::launch_fill_zero(a.accum, words, st);
+            if (e != hipSuccess) return hip_fail(e, "launch fill_zero_kernel");
+            g_static_dirty[w->device] = false;
+        }
+    } else if (int st_ws = stream_words(mw, stream, &a.accum, &slot)) {
         return st_ws;
     }
     if (cols && m > 1) {
@@ -409,7 +428,10 @@ int run_matvec(const lutgemm_weight *w, const void *x, void *y, int m, void *str
         }
         hipError_t e = lutgemm_kernels::launch_matvec(s.q, s.has_offset, s.gsub, a, plan.ntiles * plan.k_splits,
                                                       plan.waves, st);
-        if (e != hipSuccess) return hip_fail(e, "launch lut_matvec_kernel");
+        if (e != hipSuccess) {
+            if (static_ws && r > 0) g_static_dirty[w->device] = true;
+            return hip_fail(e, "launch lut_matvec_kernel");
+        }
     }
     return LUTGEMM_OK;
 }
@@ -545,7 +567,12 @@ int lutgemm_weight_info(const lutgemm_weight *w, lutgemm_weight_info_t *info)
 
 int lutgemm_matvec(const lutgemm_weight *w, const void *x, void *y, int m, void *stream)
 {
-    return run_matvec(w, x, y, m, stream, false);
+    return run_matvec(w, x, y, m, stream, false, false);
+}
+
+int lutgemm_matvec_static(const lutgemm_weight *w, const void *x, void *y, int m, void *stream)
+{
+    return run_matvec(w, x, y, m, stream, false, true);
 }
 
 int lutgemm_weight_reset_workspace(lutgemm_weight *w, void *stream)
@@ -566,7 +593,7 @@ int lutgemm_weight_reset_workspace(lutgemm_weight *w, void *stream)
 
 int lutgemm_matvec_cols(const lutgemm_weight *w, const void *x, void *y, int m, void *stream)
 {
-    return run_matvec(w, x, y, m, stream, true);
+    return run_matvec(w, x, y, m, stream, true, false);
 }
 
 int lutgemm_matvec_many(const lutgemm_weight *const *ws, const void *const *xs, void *const *ys,
@@ -575,7 +602,7 @@ int lutgemm_matvec_many(const lutgemm_weight *const *ws, const void *const *xs, 
     if (!ws || !xs || !ys || !ms) return fail(LUTGEMM_ERR_NULL_POINTER, "null argument to matvec_many");
     if (count < 0) return fail(LUTGEMM_ERR_BAD_SHAPE, "count=%d is negative", count);
     for (int i = 0; i < count; i++) {
-        int st = run_matvec(ws[i], xs[i], ys[i], ms[i], stream, false);
+        int st = run_matvec(ws[i], xs[i], ys[i], ms[i], stream, false, false);
         if (st != LUTGEMM_OK) return st;
     }
     return LUTGEMM_OK;
@@ -760,11 +787,11 @@ int lutgemm_weight_autotune(lutgemm_weight *w, void *stream)
         for (lutgemm_weight *c : copies) (rows == 2 ? c->plan2 : c->plan) = p;
         int stt = LUTGEMM_OK;
         for (int r = 0; r < 2 && stt == LUTGEMM_OK; r++)
-            stt = run_matvec(copies[turn++ % copies.size()], x, y, rows, stream, false);
+            stt = run_matvec(copies[turn++ % copies.size()], x, y, rows, stream, false, false);
         if (stt != LUTGEMM_OK) return stt;
         hipError_t he = hipEventRecord(e0, st);
         for (int r = 0; r < reps && stt == LUTGEMM_OK; r++)
-            stt = run_matvec(copies[turn++ % copies.size()], x, y, rows, stream, false);
+            stt = run_matvec(copies[turn++ % copies.size()], x, y, rows, stream, false, false);
         if (stt != LUTGEMM_OK) return stt;
         if (he == hipSuccess) he = hipEventRecord(e1, st);
         if (he == hipSuccess) he = hipEventSynchronize(e1);

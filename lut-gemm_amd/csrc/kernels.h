@@ -42,6 +42,15 @@ hipError_t launch_matvec(int q, int has_offset, int gsub, const MatvecArgs &a, i
 // words[0..count) = 0 (a fill kernel rather than a memset node, so that it can be captured)
 hipError_t launch_fill_zero(unsigned long long *words, size_t count, hipStream_t stream);
 
+// Split-k words of the allocation-free entry point: a static device array of kStaticSplitKWords
+// 64-bit words (1 MiB on every device the library runs on, enough for 65,536 outputs per
+// activation row of a two-row pass), zero at load and zero again after every completed launch.
+// Returns its device address on `device`, which must be the current device (0 <= device <
+// kMaxDevices); looked up once per device.
+constexpr size_t kStaticSplitKWords = (size_t)1 << 17;
+constexpr int kMaxDevices = 64;
+hipError_t static_split_k_words(int device, unsigned long long **words);
+
 // fp16 [k][m] -> [m][k]
 hipError_t launch_gather_columns(const void *cols, void *rows, int k, int m, hipStream_t stream);
 

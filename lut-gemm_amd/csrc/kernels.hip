@@ -24,6 +24,7 @@
 #include <hip/hip_runtime.h>
 
 #include <atomic>
+#include <mutex>
 #include <type_traits>
 #include <utility>
 
@@ -35,6 +36,10 @@ namespace lutgemm_kernels {
 using namespace lutgemm_layout;
 
 namespace {
+
+// Split-k words of the allocation-free entry point.  In host code this name is not a device
+// address, only the handle hipGetSymbolAddress takes; kernels get the address it returns.
+static __device__ __align__(256) unsigned long long scratch[kStaticSplitKWords];
 
 constexpr int kTableFloats = 256 * kLanes;  // one table set: 64 KiB
 
@@ -855,6 +860,23 @@ hipError_t launch_matvec(int q, int has_offset, int gsub, const MatvecArgs &a, i
         case 8: return launch_off<8>(has_offset, gsub, a, workgroups, th, stream);
         default: return hipErrorInvalidValue;
     }
+}
+
+hipError_t static_split_k_words(int device, unsigned long long **words)
+{
+    static std::mutex mutex;
+    static unsigned long long *address[kMaxDevices];  // each device holds its own copy of the array
+    if (device < 0 || device >= kMaxDevices) return hipErrorInvalidDevice;
+    std::lock_guard<std::mutex> lock(mutex);
+    if (!address[device]) {
+        unsigned long long *p = nullptr;
+        const hipError_t e = hipGetSymbolAddress((void **)&p, HIP_SYMBOL(scratch));
+        if (e != hipSuccess) return e;
+        if (!p) return hipErrorInvalidSymbol;
+        address[device] = p;
+    }
+    *words = address[device];
+    return hipSuccess;
 }
 
 hipError_t launch_fill_zero(unsigned long long *words, size_t count, hipStream_t stream)

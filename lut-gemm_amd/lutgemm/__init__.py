@@ -31,7 +31,7 @@ EXPORTED = [
     "lutgemm_pack_host", "lutgemm_unpack_host", "lutgemm_float_to_half", "lutgemm_last_error",
     "lutgemm_status_string", "lutgemm_version", "lutgemm_pack_file", "lutgemm_unpack_file", "lutgemm_weight_save",
     "lutgemm_weight_load", "lutgemm_weight_clone", "lutgemm_read_probe", "lutgemm_dense_gemv_f16",
-    "lutgemm_weight_reset_workspace",
+    "lutgemm_weight_reset_workspace", "lutgemm_matvec_static",
 ]
 
 
@@ -79,6 +79,7 @@ def load():
     L.lutgemm_weight_info.argtypes = [vp, ctypes.POINTER(WeightInfo)]
     L.lutgemm_matvec.argtypes = [vp, vp, vp, i, vp]
     L.lutgemm_matvec_cols.argtypes = [vp, vp, vp, i, vp]
+    L.lutgemm_matvec_static.argtypes = [vp, vp, vp, i, vp]
     L.lutgemm_matvec_many.argtypes = [vp, vp, vp, vp, i, vp]
     L.lutgemm_dequantize.argtypes = [vp, vp, i, vp]
     L.lutgemm_weight_unpack.argtypes = [vp, vp, vp, vp]
@@ -269,6 +270,10 @@ class BCQWeight:
 
     def matvec(self, x_ptr, y_ptr, m=1, stream=0):
         _check(load().lutgemm_matvec(self._h, x_ptr, y_ptr, m, stream or None))
+
+    def matvec_static(self, x_ptr, y_ptr, m=1, stream=0):
+        """matvec with the split-k words in the library's static device array: allocates nothing."""
+        _check(load().lutgemm_matvec_static(self._h, x_ptr, y_ptr, m, stream or None))
 
     def matvec_cols(self, x_ptr, y_ptr, m=1, stream=0):
         _check(load().lutgemm_matvec_cols(self._h, x_ptr, y_ptr, m, stream or None))
