@@ -42,7 +42,7 @@ METRIC = "µs/matvec + weight-GB/s (% HBM peak), n=k=12288 q=3 g=128 m=1 fp16"
 # profiles/lut_matvec_kernel_cfg1.md (FETCH_SIZE and WRITE_SIZE, scaled by the factors a plain
 # copy kernel of known size reads on the same counters)
 # (64.01 MB read for either plan; 0.91 MB written with 8 k-splits, 0.61 MB with 5: fewer split-k atomics)
-CFG1_MEASURED_TRAFFIC_BYTES = {8: 64.9e6, 5: 64.6e6}  # by k-splits of the launch plan
+CFG1_MEASURED_TRAFFIC_BYTES_PER_MATVEC = None  # set from the counter runs of the fused kernel (profiles/)
 
 
 def event_time_ms(torch, fn, stream):
@@ -170,7 +170,7 @@ class Point:
             wgt.close()
 
 
-PREWARM_MS = 40.0   # the device reaches its sustained clocks only after some tens of ms under load
+PREWARM_MS = 100.0  # the device reaches its sustained clocks only after some tens of ms under load
 BURSTS = 15         # the --steps burst is timed this many times back to back; the median is reported
 
 
@@ -202,25 +202,32 @@ def median(v):
 
 
 def time_point(lutgemm, torch, stream, pt, steps, warmup):
-    """us per step, rotating copies and single copy: `warmup` untimed steps, then (whatever
-    `warmup` is) PREWARM_MS of launches so that the clocks are up, then BURSTS bursts of exactly
-    `steps` steps; the median burst counts.  The rotation over the weight copies continues from
-    burst to burst, so no burst finds its weights in the memory-side cache."""
+    """us per step with one launch per matvec (rotating copies and single copy): `warmup` untimed
+    steps, then (whatever `warmup` is) PREWARM_MS of launches so that the clocks are up, then
+    BURSTS bursts of exactly `steps` steps; the median burst counts.  The rotation over the weight
+    copies continues from burst to burst, so no burst finds its weights in the memory-side cache.
+    pt.fused_us: the same bursts through lutgemm_matvec_many, which puts up to sixteen independent
+    matvecs (here: different weight copies) into one launch."""
     sh = stream.cuda_stream
-    lutgemm.MatvecSequence(pt.items(max(1, warmup))).launch(sh)
+    lutgemm.MatvecSequence(pt.items(max(1, warmup))).launch(sh, fused=False)
     torch.cuda.synchronize()
     seqs = [lutgemm.MatvecSequence(pt.items(steps, offset=b * steps)) for b in range(BURSTS)]
     hot = lutgemm.MatvecSequence(pt.items(steps, rotate=False))
-    prewarm(torch, lambda: seqs[0].launch(sh))
-    ms = time_bursts(torch, stream, [(lambda q=q: q.launch(sh)) for q in seqs])
-    ms_hot = time_bursts(torch, stream, [lambda: hot.launch(sh)] * BURSTS)
+    prewarm(torch, lambda: seqs[0].launch(sh, fused=False))
+    ms = time_bursts(torch, stream, [(lambda q=q: q.launch(sh, fused=False)) for q in seqs])
+    ms_hot = time_bursts(torch, stream, [lambda: hot.launch(sh, fused=False)] * BURSTS)
+    ms_fused = time_bursts(torch, stream, [(lambda q=q: q.launch(sh, fused=True)) for q in seqs])
     pt.burst_us = [t * 1e3 / steps for t in ms]
+    pt.fused_burst_us = [t * 1e3 / steps for t in ms_fused]
+    pt.fused_us = median(ms_fused) * 1e3 / steps
     return median(ms) * 1e3 / steps, median(ms_hot) * 1e3 / steps
 
 
 def point_record(pt, us, us_hot):
     return {"k": pt.k, "n": pt.n, "q": pt.q, "g": pt.g, "m": pt.m, "offset": pt.has_offset,
             "us_per_matvec": us, "weight_GBps": pt.b_w / us / 1e3, "pct_hbm_peak": pt.b_w / us / 1e3 / HBM_PEAK_GBS * 100,
+            "fused_independent_us_per_matvec": pt.fused_us,
+            "fused_independent_pct_hbm_peak": pt.b_w / pt.fused_us / 1e3 / HBM_PEAK_GBS * 100,
             "hot_us_per_matvec": us_hot, "packed_weight_bytes": pt.b_w, "weight_copies_rotated": pt.copies,
             "plan": pt.plan}
 
@@ -239,12 +246,16 @@ def base_line(args, metric, value, us, workload, extra_config=None):
     }
 
 
+MAX_FUSED = 32   # independent matvecs lutgemm_matvec_many puts into one launch
+
+
 def run_single(args, lutgemm, synth, torch, dev, stream, name):
     cfg = synth.CONFIGS[name]
     k, n, q, g = cfg["k"], cfg["n"], cfg["q"], cfg["g"]
     pt = Point(lutgemm, synth, torch, dev, k, n, q, g, cfg["rtn"], 1, 1, stream.cuda_stream,
                copies=args.copies if name == "cfg1" else None, plan=args.plan)
-    us, us_hot = time_point(lutgemm, torch, stream, pt, args.steps, args.warmup)
+    us_each, us_hot = time_point(lutgemm, torch, stream, pt, args.steps, args.warmup)
+    us = pt.fused_us     # the steps are independent matvecs: whole-job throughput through lutgemm_matvec_many
     weight_gbs = pt.b_w / (us * 1e-6) / 1e9
     achieved = pt.b_total / (us * 1e-6) / 1e9
     parity, truth = pt.parity(None if name != "cfg2" else 4096)
@@ -252,20 +263,33 @@ def run_single(args, lutgemm, synth, torch, dev, stream, name):
     metric = METRIC if name == "cfg1" else "µs/matvec + weight-GB/s (%% HBM peak), k=%d n=%d q=%d g=%d m=1 fp16" % (k, n, q, g)
     workload = "%s: BCQ matvec m=1 k=%d n=%d q=%d g=%d %s" % (
         name, k, n, q, g, "RTN codes as BCQ with offset" if cfg["rtn"] else "no offset")
+    units = min(args.steps, MAX_FUSED, pt.copies)
     line = base_line(args, metric, weight_gbs, us, workload,
-                     {"weight_copies_rotated": pt.copies, "packed_weight_bytes": pt.b_w, "plan": pt.plan})
+                     {"weight_copies_rotated": pt.copies, "packed_weight_bytes": pt.b_w,
+                      "launch": "the %d steps of a burst are independent matvecs (one weight copy each) issued with one "
+                                "lutgemm_matvec_many call, which puts up to %d of them into one kernel launch" % (args.steps, MAX_FUSED),
+                      "plan_of_single_launches": pt.plan})
     line["ms_per_step"] = us / 1e3
-    kernel = "lut_matvec_kernel<%d,%s,1>" % (q, "true" if pt.has_offset else "false")
-    traffic = CFG1_MEASURED_TRAFFIC_BYTES.get(pt.plan["k_splits"]) if name == "cfg1" else None
+    kernel = "lut_matvec_multi_kernel<%d,%s,1>" % (q, "true" if pt.has_offset else "false")
+    traffic_unit = CFG1_MEASURED_TRAFFIC_BYTES_PER_MATVEC if name == "cfg1" else None
     line["roofline"] = {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                        "frac": achieved / HBM_PEAK_GBS, "traffic": traffic,
+                        "frac": achieved / HBM_PEAK_GBS,
+                        "traffic": traffic_unit * units if traffic_unit is not None else None,
                         "traffic_source": (
-                            "not measured in this run: rocprofv3 --pmc FETCH_SIZE x 2.000 + WRITE_SIZE x 1.000 per dispatch for "
-                            "this launch plan, from profiles/lut_matvec_kernel_cfg1.md" if traffic is not None else
-                            "no counter run on record for this workload and launch plan (profiles/)"),
-                        "kernel": kernel, "algorithmic_bytes_per_launch": pt.b_total, "avg_launch_us": us,
-                        "launch_us_bursts": pt.burst_us}
-    line["hot_single_copy"] = {"us_per_matvec": us_hot, "weight_GBps": pt.b_w / (us_hot * 1e-6) / 1e9}
+                            "not measured in this run: rocprofv3 --pmc FETCH_SIZE x 2.000 + WRITE_SIZE x 1.000 per dispatch of "
+                            "this kernel divided by the matvecs of the dispatch, from profiles/lut_matvec_multi_kernel_cfg1.md, "
+                            "times the matvecs per launch of this run" if traffic_unit is not None else
+                            "no counter run on record for this workload (profiles/)"),
+                        "kernel": kernel, "matvecs_per_launch": units,
+                        "algorithmic_bytes_per_launch": pt.b_total * units, "avg_launch_us": us * units,
+                        "us_per_matvec_bursts": pt.fused_burst_us}
+    line["one_launch_per_matvec"] = {
+        "what": "the same bursts with one kernel launch per matvec (lutgemm_matvec_each): what a chain of matvecs that "
+                "depend on each other sees; every launch pays its own start, end and launch gap",
+        "kernel": "lut_matvec_kernel<%d,%s,1>" % (q, "true" if pt.has_offset else "false"), "plan": pt.plan,
+        "us_per_matvec": us_each, "weight_GBps": pt.b_w / us_each / 1e3,
+        "roofline_frac": pt.b_total / us_each / 1e3 / HBM_PEAK_GBS, "us_per_matvec_bursts": pt.burst_us,
+        "hot_single_copy_us_per_matvec": us_hot}
     # the device's pure-read time for the same tiles, same grid, same rotation over the copies,
     # timed like the matvec (clocks warmed, median of BURSTS bursts)
     reads = max(1, args.steps)
@@ -274,9 +298,10 @@ def run_single(args, lutgemm, synth, torch, dev, stream, name):
     rms = time_bursts(torch, stream, [(lambda o=o: lutgemm.read_probe(o, stream.cuda_stream)) for o in orders])
     read_us = median(rms) * 1e3 / reads
     tile_bytes = sum(lutgemm.packed_sizes(k, n, q, k // g, pt.has_offset))  # packed tiles incl. padding
-    line["pure_read_same_tiles"] = {"us": read_us, "bytes": tile_bytes, "GBps": tile_bytes / read_us / 1e3,
-                                    "matvec_time_over_read_time": us / read_us}
-    line["roofline"]["read_floor_us"] = read_us
+    line["one_launch_per_matvec"]["pure_read_same_tiles"] = {
+        "what": "one launch per weight that only reads the tiles (same grid, same loads in flight): the floor of a single launch",
+        "us": read_us, "bytes": tile_bytes, "GBps": tile_bytes / read_us / 1e3, "matvec_time_over_read_time": us_each / read_us}
+    line["roofline"]["read_floor_us_single_launch"] = read_us
     if name == "cfg1":
         import numpy as np
         from oracle import oracle
@@ -316,7 +341,7 @@ def run_single(args, lutgemm, synth, torch, dev, stream, name):
         dense = {"kind": "torch.mv fp16 (rocBLAS/hipBLASLt)", "us_per_matvec": dense_us,
                  "bytes": 2 * k * n + 2 * k + 2 * n,
                  "GBps": (2 * k * n + 2 * k + 2 * n) / (dense_us * 1e-6) / 1e9,
-                 "lut_speedup": dense_us / us}
+                 "lut_speedup": dense_us / us, "lut_speedup_one_launch_per_matvec": dense_us / us_each}
         # the same product through this library's plain streaming kernel (bandwidth-bound comparator)
         sh = stream.cuda_stream
         for i in range(10):
@@ -329,7 +354,8 @@ def run_single(args, lutgemm, synth, torch, dev, stream, name):
                 lutgemm.dense_gemv(Wd[i % nd].data_ptr(), xv.data_ptr(), outs[i % nd].data_ptr(), k, n, sh)
         pus = event_time_ms(torch, run_plain, stream) * 1e3 / reps
         dense["handwritten_streaming_gemv"] = {"us_per_matvec": pus, "GBps": dense["bytes"] / pus / 1e3,
-                                                "lut_speedup": pus / us, "agrees_with_library": agree}
+                                                "lut_speedup": pus / us, "lut_speedup_one_launch_per_matvec": pus / us_each,
+                                                "agrees_with_library": agree}
         del Wd
     line["dense_fp16_gemv"] = dense
     line["cpu_baseline"] = None
@@ -341,7 +367,7 @@ def run_single(args, lutgemm, synth, torch, dev, stream, name):
 
 def run_cfg3(args, lutgemm, synth, torch, dev, stream):
     points = []
-    tot_bytes = tot_us = 0.0
+    tot_bytes = tot_us = tot_fused = 0.0
     worst = 0.0
     for c in synth.CFG3_POINTS:
         pt = Point(lutgemm, synth, torch, dev, c["k"], c["n"], c["q"], c["g"], False, 1, c["q"] * 10000 + c["g"],
@@ -353,16 +379,20 @@ def run_cfg3(args, lutgemm, synth, torch, dev, stream):
         points.append(rec)
         tot_bytes += pt.b_w
         tot_us += us
+        tot_fused += pt.fused_us
         pt.close()
-    value = tot_bytes / tot_us / 1e3
+    value = tot_bytes / tot_fused / 1e3
     line = base_line(args, "weight-GB/s over the k=n=7168 sweep (q 1..4 x g 32,64,128,k), m=1 fp16", value,
-                     tot_us / len(points), "cfg3: 16 BCQ matvecs k=n=7168, q in 1..4, g in {32,64,128,7168}",
-                     {"points": len(points)})
-    line["ms_per_step"] = tot_us / 1e3
+                     tot_fused / len(points), "cfg3: 16 BCQ matvecs k=n=7168, q in 1..4, g in {32,64,128,7168}",
+                     {"points": len(points),
+                      "launch": "per point, bursts of independent matvecs (one weight copy each) through lutgemm_matvec_many"})
+    line["ms_per_step"] = tot_fused / 1e3
     line["points"] = points
+    line["one_launch_per_matvec"] = {"weight_GBps": tot_bytes / tot_us / 1e3, "us_sum": tot_us,
+                                     "frac_hbm_peak": tot_bytes / tot_us / 1e3 / HBM_PEAK_GBS}
     line["parity"] = {"worst_max_abs": worst, "outputs_checked_per_point": 2048}
     line["roofline"] = {"bound": "hbm", "achieved": value, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                        "frac": value / HBM_PEAK_GBS, "traffic": None, "kernel": "lut_matvec_kernel<q,false,gsub>",
+                        "frac": value / HBM_PEAK_GBS, "traffic": None, "kernel": "lut_matvec_multi_kernel<q,false,gsub>",
                         "note": "aggregate packed-weight bytes / summed time over the 16 points"}
     line["cpu_baseline"] = None
     return line
@@ -394,11 +424,12 @@ def run_cfg4(args, lutgemm, synth, torch, dev, stream):
                 out.extend(pts[nm].items(1, offset=s))
         return out
 
-    lutgemm.MatvecSequence(chain_items(max(1, args.warmup))).launch(sh)
+    # a decoder's projections depend on each other: one launch per matvec, in order
+    lutgemm.MatvecSequence(chain_items(max(1, args.warmup))).launch(sh, fused=False)
     torch.cuda.synchronize()
     timed = lutgemm.MatvecSequence(chain_items(args.steps))
-    prewarm(torch, lambda: timed.launch(sh))
-    ms = median(time_bursts(torch, stream, [lambda: timed.launch(sh)] * 7))
+    prewarm(torch, lambda: timed.launch(sh, fused=False))
+    ms = median(time_bursts(torch, stream, [lambda: timed.launch(sh, fused=False)] * 7))
     chain_us = ms * 1e3 / args.steps
     graph = None
     if args.graph:
@@ -410,10 +441,10 @@ def run_cfg4(args, lutgemm, synth, torch, dev, stream):
         side = torch.cuda.Stream()
         side.wait_stream(stream)
         with torch.cuda.stream(side):
-            seq.launch(side.cuda_stream)  # warm-up on the capture stream
+            seq.launch(side.cuda_stream, fused=False)  # warm-up on the capture stream
             side.synchronize()
             with torch.cuda.graph(g, stream=side):
-                seq.launch(torch.cuda.current_stream().cuda_stream)
+                seq.launch(torch.cuda.current_stream().cuda_stream, fused=False)
         stream.wait_stream(side)
         torch.cuda.synchronize()
         reps = max(1, args.steps // copies)
@@ -514,7 +545,7 @@ def main():
     ap.add_argument("--config", default="cfg1", choices=["cfg0", "cfg1", "cfg2", "cfg3", "cfg4", "dequant"])
     ap.add_argument("--m", type=int, default=1, help="activation rows (cfg4 only)")
     ap.add_argument("--graph", action="store_true", help="cfg4: also replay the chain from a captured HIP graph")
-    ap.add_argument("--copies", type=int, default=17, help="cfg1: distinct weight copies rotated through")
+    ap.add_argument("--copies", type=int, default=33, help="cfg1: distinct weight copies rotated through")
     ap.add_argument("--plan", default=None,
                     help="cfg0/1/2: WAVES,KSPLITS launch plan instead of the measured choice (profiling runs)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")

@@ -129,6 +129,54 @@ Plan choose_plan(const Shape &s, int cus)
     return best;
 }
 
+// Launch shape of several independent one-row matvecs in one grid (lutgemm_matvec_many): one
+// number of wavefronts per workgroup and one number of k-blocks per workgroup for all entries.
+// A compute unit holds one workgroup at a time (its table sets take most of the LDS), so a unit
+// works through its workgroups one after the other and pays for each its start (first memory
+// round trip, first table) and its end (reduction, split-k atomic) in full; what the single grid
+// removes is the idle time of the memory system: while one unit is between workgroups the others
+// stream.  The grid runs in rounds of one workgroup per unit; a last round that does not fill
+// the device streams faster per workgroup, but less than proportionally.  Long workgroups amortise
+// start and end, short ones leave a smaller last round.  Constants (microseconds, bytes) fitted
+// to measured times of 40 plans over five weight shapes and run lengths 3 to 32 on MI355X.
+struct FusedPlan { int waves, blocks_per_group; };
+
+FusedPlan choose_fused_plan(const Shape *const *shapes, int count, int cus)
+{
+    const double kBytesPerCu = 7.0e6 / 256.0;  // streaming rate per compute unit with all units busy
+    const double kBlockFloor = 1.7;            // a k-block takes at least one loaded memory round trip
+    const double kStartEnd = 2.4, kStartEndPerWave = 0.17;  // per workgroup: 2.4 at 12 wavefronts, more with fewer
+    const double kPartialExponent = 0.28;      // a round on a fraction f of the units streams f^0.28 as long
+    int max_ts = 1;
+    for (int e = 0; e < count; e++) max_ts = shapes[e]->ts > max_ts ? shapes[e]->ts : max_ts;
+    FusedPlan best{kMaxWaves, max_ts};
+    double best_cost = 1e300;
+    for (int waves = 1; waves <= kMaxWaves; waves++)
+        for (int bpg = div_up(max_ts, kMaxSplits); bpg <= max_ts; bpg++) {
+            long groups = 0;
+            double stream = 0.0;  // summed streaming time of all workgroups
+            for (int e = 0; e < count; e++) {
+                const Shape &s = *shapes[e];
+                const int b = bpg < s.ts ? bpg : s.ts;
+                const long g = (long)div_up(s.nb, waves) * div_up(s.ts, b);
+                double t_block = waves * (double)(sign_tile_bytes(s) + scale_tile_bytes(s)) / kBytesPerCu;
+                if (t_block < kBlockFloor) t_block = kBlockFloor;
+                groups += g;
+                stream += (double)g * b * t_block;
+            }
+            const double per_group = stream / (double)groups;
+            const double start_end = kStartEnd + kStartEndPerWave * (kMaxWaves - waves);
+            const long full = groups / cus, rest = groups % cus;
+            double cost = (double)full * (per_group + start_end);
+            if (rest) cost += per_group * std::pow((double)rest / cus, kPartialExponent) + start_end;
+            if (cost < best_cost - 1e-9) {
+                best_cost = cost;
+                best = FusedPlan{waves, bpg};
+            }
+        }
+    return best;
+}
+
 // A handle's device memory belongs to the device that was current when it was created.
 int check_device(const lutgemm_weight *w)
 {
@@ -596,14 +644,88 @@ int lutgemm_matvec_cols(const lutgemm_weight *w, const void *x, void *y, int m, 
     return run_matvec(w, x, y, m, stream, true, false);
 }
 
+int lutgemm_matvec_each(const lutgemm_weight *const *ws, const void *const *xs, void *const *ys,
+                        const int *ms, int count, void *stream)
+{
+    if (!ws || !xs || !ys || !ms) return fail(LUTGEMM_ERR_NULL_POINTER, "null argument to matvec_each");
+    if (count < 0) return fail(LUTGEMM_ERR_BAD_SHAPE, "count=%d is negative", count);
+    for (int i = 0; i < count; i++) {
+        int st = run_matvec(ws[i], xs[i], ys[i], ms[i], stream, false, false);
+        if (st != LUTGEMM_OK) return st;
+    }
+    return LUTGEMM_OK;
+}
+
 int lutgemm_matvec_many(const lutgemm_weight *const *ws, const void *const *xs, void *const *ys,
                         const int *ms, int count, void *stream)
 {
     if (!ws || !xs || !ys || !ms) return fail(LUTGEMM_ERR_NULL_POINTER, "null argument to matvec_many");
     if (count < 0) return fail(LUTGEMM_ERR_BAD_SHAPE, "count=%d is negative", count);
-    for (int i = 0; i < count; i++) {
-        int st = run_matvec(ws[i], xs[i], ys[i], ms[i], stream, false, false);
-        if (st != LUTGEMM_OK) return st;
+    struct Range { uintptr_t lo, hi; };
+    auto overlap = [](const Range &a, const Range &b) { return a.lo < b.hi && b.lo < a.hi; };
+    int i = 0;
+    while (i < count) {
+        // Longest run of entries starting at i that one launch can take: one activation row each,
+        // the same kernel instance, no handle twice (its split-k words would be shared), and no
+        // output overlapping an input or output of another entry of the run, so that their order
+        // does not matter.  Anything else goes through its own launch, in order.
+        lutgemm_kernels::MultiMatvecArgs multi{};
+        Range xr[lutgemm_kernels::kMaxFused], yr[lutgemm_kernels::kMaxFused];
+        const Shape *shapes[lutgemm_kernels::kMaxFused];
+        int j = i;
+        const lutgemm_weight *w0 = ws[i];
+        for (; j < count && j - i < lutgemm_kernels::kMaxFused; j++) {
+            const lutgemm_weight *w = ws[j];
+            if (!w || !xs[j] || !ys[j] || ms[j] != 1 || ((uintptr_t)xs[j] & 15u) != 0) break;
+            const Shape &s = w->shape;
+            if (s.q != w0->shape.q || s.has_offset != w0->shape.has_offset || s.gsub != w0->shape.gsub ||
+                w->device != w0->device)
+                break;
+            const int e = j - i;
+            xr[e] = Range{(uintptr_t)xs[j], (uintptr_t)xs[j] + (size_t)s.k * 2};
+            yr[e] = Range{(uintptr_t)ys[j], (uintptr_t)ys[j] + (size_t)s.n * 2};
+            bool independent = true;
+            for (int p = 0; p < e && independent; p++)
+                independent = ws[i + p] != w && !overlap(yr[e], yr[p]) && !overlap(yr[e], xr[p]) && !overlap(xr[e], yr[p]);
+            if (!independent) break;
+            shapes[e] = &s;
+            lutgemm_kernels::MatvecArgs &a = multi.entry[e];
+            a.signs = w->d_signs;
+            a.scales = w->d_scales;
+            a.k = s.k;
+            a.n = s.n;
+            a.ts = s.ts;
+            a.nb = s.nb;
+            a.x = xs[j];
+            a.y = ys[j];
+            a.y_stride = 1;
+            a.rows = 1;
+        }
+        const int run = j - i;
+        if (run < 2) {
+            int st = run_matvec(ws[i], xs[i], ys[i], ms[i], stream, false, false);
+            if (st != LUTGEMM_OK) return st;
+            i++;
+            continue;
+        }
+        if (int st_dev = check_device(w0)) return st_dev;
+        const FusedPlan fp = choose_fused_plan(shapes, run, w0->compute_units);
+        int blocks = 0;
+        for (int e = 0; e < run; e++) {
+            lutgemm_kernels::MatvecArgs &a = multi.entry[e];
+            a.ntiles = div_up(a.nb, fp.waves);
+            a.blocks_per_split = fp.blocks_per_group < a.ts ? fp.blocks_per_group : a.ts;
+            a.k_splits = div_up(a.ts, a.blocks_per_split);
+            multi.first_block[e] = blocks;
+            blocks += a.ntiles * a.k_splits;
+            int slot = 0;
+            if (int st_ws = stream_words(const_cast<lutgemm_weight *>(ws[i + e]), stream, &a.accum, &slot)) return st_ws;
+        }
+        multi.count = run;
+        hipError_t e = lutgemm_kernels::launch_matvec_multi(w0->shape.q, w0->shape.has_offset, w0->shape.gsub, multi,
+                                                            blocks, fp.waves, static_cast<hipStream_t>(stream));
+        if (e != hipSuccess) return hip_fail(e, "launch lut_matvec_multi_kernel");
+        i = j;
     }
     return LUTGEMM_OK;
 }

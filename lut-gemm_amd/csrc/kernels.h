@@ -27,6 +27,15 @@ struct MatvecArgs {
     long long x_row_stride, y_row_stride, accum_row_stride;
 };
 
+// Up to kMaxFused independent one-row matvecs for one launch: entry i owns the workgroups
+// first_block[i] .. first_block[i+1]-1 of the grid (the last entry up to the end).
+constexpr int kMaxFused = 32;
+struct MultiMatvecArgs {
+    int count;
+    int first_block[kMaxFused];
+    MatvecArgs entry[kMaxFused];
+};
+
 struct DequantArgs {
     const uint8_t *signs;
     const uint16_t *scales;
@@ -38,6 +47,10 @@ struct DequantArgs {
 // workgroups = ntiles * k_splits, `waves` wavefronts of 64 lanes per workgroup.
 hipError_t launch_matvec(int q, int has_offset, int gsub, const MatvecArgs &a, int workgroups,
                          int waves, hipStream_t stream);
+
+// entries with rows == 1 sharing q, has_offset, gsub and the wavefronts per workgroup
+hipError_t launch_matvec_multi(int q, int has_offset, int gsub, const MultiMatvecArgs &m, int workgroups, int waves,
+                               hipStream_t stream);
 
 // words[0..count) = 0 (a fill kernel rather than a memset node, so that it can be captured)
 hipError_t launch_fill_zero(unsigned long long *words, size_t count, hipStream_t stream);

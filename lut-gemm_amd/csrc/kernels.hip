@@ -535,8 +535,9 @@ __device__ __forceinline__ void finish_output(float total, bool active, int out,
     }
 }
 
+// Workgroup `block` of one matvec (the body of lut_matvec_kernel and of lut_matvec_multi_kernel).
 template <int Q, bool OFF, int GSUB>
-__global__ __launch_bounds__(768) void lut_matvec_kernel(MatvecArgs a)
+__device__ __forceinline__ void matvec_workgroup(const MatvecArgs &a, int block)
 {
     constexpr int QO = Q + (OFF ? 1 : 0);
     // Two table sets: while the lookups of k-block t read one, the other is rebuilt for t+1.
@@ -548,8 +549,8 @@ __global__ __launch_bounds__(768) void lut_matvec_kernel(MatvecArgs a)
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform by construction
     const int waves = blockDim.x >> 6;
-    const int ntile = blockIdx.x % a.ntiles;
-    const int ks = blockIdx.x / a.ntiles;
+    const int ntile = block % a.ntiles;
+    const int ks = block / a.ntiles;
     const int nb = ntile * waves + wave;
     const bool active = nb < a.nb;
     const int ts0 = ks * a.blocks_per_split;
@@ -614,6 +615,24 @@ __global__ __launch_bounds__(768) void lut_matvec_kernel(MatvecArgs a)
 
     const float total = reduce_across_lanes(acc, lane);
     finish_output(total, active, nb * kBatch + (lane >> 1), lane, reinterpret_cast<__half *>(a.y), a.accum, a);
+}
+
+template <int Q, bool OFF, int GSUB>
+__global__ __launch_bounds__(768) void lut_matvec_kernel(MatvecArgs a)
+{
+    matvec_workgroup<Q, OFF, GSUB>(a, blockIdx.x);
+}
+
+// Several independent one-row matvecs in one launch: the workgroups of entry i follow those of
+// entry i-1 in the grid, so a compute unit that has finished its share of one matvec starts on the
+// next while other units are still at the end of theirs, and the matvecs pay one launch between
+// them instead of one each.  All entries share Q, OFF, GSUB and the wavefronts per workgroup.
+template <int Q, bool OFF, int GSUB>
+__global__ __launch_bounds__(768) void lut_matvec_multi_kernel(MultiMatvecArgs m)
+{
+    int i = 0;
+    while (i + 1 < m.count && (int)blockIdx.x >= m.first_block[i + 1]) i++;   // scalar: at most 31 steps
+    matvec_workgroup<Q, OFF, GSUB>(m.entry[i], (int)blockIdx.x - m.first_block[i]);
 }
 
 // process_tile for two activation rows (tables of lookup8x2).
@@ -799,6 +818,23 @@ __global__ __launch_bounds__(256) void fill_zero_kernel(unsigned long long *word
         words[i] = 0ull;
 }
 
+// more than 64 KiB of dynamic LDS has to be allowed once per kernel and device
+template <typename Kernel>
+hipError_t allow_two_table_sets(Kernel kernel, std::atomic<unsigned long long> &allowed)
+{
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return e;
+    const unsigned long long bit = 1ull << (dev & 63);
+    if (!(allowed.load(std::memory_order_relaxed) & bit)) {
+        e = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                2 * kTableFloats * (int)sizeof(float));
+        if (e != hipSuccess) return e;
+        allowed.fetch_or(bit, std::memory_order_relaxed);
+    }
+    return hipSuccess;
+}
+
 template <int Q, bool OFF, int GSUB>
 hipError_t launch_one(const MatvecArgs &a, int workgroups, int threads, hipStream_t stream)
 {
@@ -808,22 +844,25 @@ hipError_t launch_one(const MatvecArgs &a, int workgroups, int threads, hipStrea
         hipLaunchKernelGGL((lut_matvec2_kernel<Q, OFF, GSUB>), dim3(workgroups), dim3(threads), 0, stream, a);
     else
     {
-        // more than 64 KiB of dynamic LDS has to be allowed once per kernel and device
         static std::atomic<unsigned long long> allowed{0};
-        int dev = 0;
-        hipError_t e = hipGetDevice(&dev);
+        const hipError_t e = allow_two_table_sets(&lut_matvec_kernel<Q, OFF, GSUB>, allowed);
         if (e != hipSuccess) return e;
-        const unsigned long long bit = 1ull << (dev & 63);
-        if (!(allowed.load(std::memory_order_relaxed) & bit)) {
-            e = hipFuncSetAttribute(reinterpret_cast<const void *>(&lut_matvec_kernel<Q, OFF, GSUB>),
-                                    hipFuncAttributeMaxDynamicSharedMemorySize,
-                                    2 * kTableFloats * (int)sizeof(float));
-            if (e != hipSuccess) return e;
-            allowed.fetch_or(bit, std::memory_order_relaxed);
-        }
         const size_t lds = (size_t)(a.blocks_per_split == 1 ? 1 : 2) * kTableFloats * sizeof(float);
         hipLaunchKernelGGL((lut_matvec_kernel<Q, OFF, GSUB>), dim3(workgroups), dim3(threads), lds, stream, a);
     }
+    return hipGetLastError();
+}
+
+template <int Q, bool OFF, int GSUB>
+hipError_t launch_multi_one(const MultiMatvecArgs &m, int workgroups, int threads, hipStream_t stream)
+{
+    static std::atomic<unsigned long long> allowed{0};
+    const hipError_t e = allow_two_table_sets(&lut_matvec_multi_kernel<Q, OFF, GSUB>, allowed);
+    if (e != hipSuccess) return e;
+    bool one_block = true;
+    for (int i = 0; i < m.count; i++) one_block = one_block && m.entry[i].blocks_per_split == 1;
+    const size_t lds = (size_t)(one_block ? 1 : 2) * kTableFloats * sizeof(float);
+    hipLaunchKernelGGL((lut_matvec_multi_kernel<Q, OFF, GSUB>), dim3(workgroups), dim3(threads), lds, stream, m);
     return hipGetLastError();
 }
 
@@ -877,6 +916,42 @@ hipError_t static_split_k_words(int device, unsigned long long **words)
     }
     *words = address[device];
     return hipSuccess;
+}
+
+namespace {
+template <int Q>
+hipError_t launch_multi_q(int has_offset, int gsub, const MultiMatvecArgs &m, int wg, int th, hipStream_t s)
+{
+    if (has_offset) {
+        switch (gsub) {
+            case 1: return launch_multi_one<Q, true, 1>(m, wg, th, s);
+            case 2: return launch_multi_one<Q, true, 2>(m, wg, th, s);
+            default: return launch_multi_one<Q, true, 4>(m, wg, th, s);
+        }
+    }
+    switch (gsub) {
+        case 1: return launch_multi_one<Q, false, 1>(m, wg, th, s);
+        case 2: return launch_multi_one<Q, false, 2>(m, wg, th, s);
+        default: return launch_multi_one<Q, false, 4>(m, wg, th, s);
+    }
+}
+}  // namespace
+
+hipError_t launch_matvec_multi(int q, int has_offset, int gsub, const MultiMatvecArgs &m, int workgroups, int waves,
+                               hipStream_t stream)
+{
+    const int th = waves * kLanes;
+    switch (q) {
+        case 1: return launch_multi_q<1>(has_offset, gsub, m, workgroups, th, stream);
+        case 2: return launch_multi_q<2>(has_offset, gsub, m, workgroups, th, stream);
+        case 3: return launch_multi_q<3>(has_offset, gsub, m, workgroups, th, stream);
+        case 4: return launch_multi_q<4>(has_offset, gsub, m, workgroups, th, stream);
+        case 5: return launch_multi_q<5>(has_offset, gsub, m, workgroups, th, stream);
+        case 6: return launch_multi_q<6>(has_offset, gsub, m, workgroups, th, stream);
+        case 7: return launch_multi_q<7>(has_offset, gsub, m, workgroups, th, stream);
+        case 8: return launch_multi_q<8>(has_offset, gsub, m, workgroups, th, stream);
+        default: return hipErrorInvalidValue;
+    }
 }
 
 hipError_t launch_fill_zero(unsigned long long *words, size_t count, hipStream_t stream)

@@ -31,7 +31,7 @@ EXPORTED = [
     "lutgemm_pack_host", "lutgemm_unpack_host", "lutgemm_float_to_half", "lutgemm_last_error",
     "lutgemm_status_string", "lutgemm_version", "lutgemm_pack_file", "lutgemm_unpack_file", "lutgemm_weight_save",
     "lutgemm_weight_load", "lutgemm_weight_clone", "lutgemm_read_probe", "lutgemm_dense_gemv_f16",
-    "lutgemm_weight_reset_workspace", "lutgemm_matvec_static",
+    "lutgemm_weight_reset_workspace", "lutgemm_matvec_static", "lutgemm_matvec_each",
 ]
 
 
@@ -81,6 +81,7 @@ def load():
     L.lutgemm_matvec_cols.argtypes = [vp, vp, vp, i, vp]
     L.lutgemm_matvec_static.argtypes = [vp, vp, vp, i, vp]
     L.lutgemm_matvec_many.argtypes = [vp, vp, vp, vp, i, vp]
+    L.lutgemm_matvec_each.argtypes = [vp, vp, vp, vp, i, vp]
     L.lutgemm_dequantize.argtypes = [vp, vp, i, vp]
     L.lutgemm_weight_unpack.argtypes = [vp, vp, vp, vp]
     L.lutgemm_weight_plan.argtypes = [vp, pi, pi, pi, pi]
@@ -307,7 +308,9 @@ def matmul(output_ptr, input_ptr, weight, m=1, stream=0):
 
 
 class MatvecSequence:
-    """A fixed list of (weight, x_ptr, y_ptr, m) issued with one lutgemm_matvec_many call."""
+    """A fixed list of (weight, x_ptr, y_ptr, m) issued with one lutgemm_matvec_many call
+    (independent neighbours share launches) or, with fused=False, one lutgemm_matvec_each call
+    (one launch per entry)."""
 
     def __init__(self, items):
         n = len(items)
@@ -318,8 +321,9 @@ class MatvecSequence:
         self._ys = (ctypes.c_void_p * n)(*[it[2] for it in items])
         self._ms = (ctypes.c_int * n)(*[it[3] for it in items])
 
-    def launch(self, stream=0):
-        _check(load().lutgemm_matvec_many(self._ws, self._xs, self._ys, self._ms, self.count, stream or None))
+    def launch(self, stream=0, fused=True):
+        fn = load().lutgemm_matvec_many if fused else load().lutgemm_matvec_each
+        _check(fn(self._ws, self._xs, self._ys, self._ms, self.count, stream or None))
 
 
 def read_probe(weights, stream=0):

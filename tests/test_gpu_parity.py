@@ -335,6 +335,76 @@ def test_non_finite_activations(lutgemm, device):
     W.close()
 
 
+def test_matvec_many_shares_launches_and_keeps_every_result(lutgemm, oracle, device):
+    """lutgemm_matvec_many puts independent neighbours into one launch with a launch shape of its
+    own (another split along k, so the last bit may differ from a lutgemm_matvec call).  Whatever
+    it decides: every entry is within the tolerance of the path against the oracle, the call is
+    deterministic, and entries that cannot share a launch (a handle that appears twice in a row, a
+    batch, an entry that reads the previous entry's output) come out bit for bit as their own
+    lutgemm_matvec call does.  Runs of equal and of different shapes, more entries than one launch
+    takes."""
+    import torch
+    from lutgemm import synth
+    st = torch.cuda.current_stream().cuda_stream
+    shapes = [(2048, 2048, 3, 128, False), (2048, 1000, 3, 128, False), (4096, 2048, 3, 256, False),
+              (2048, 2048, 3, 64, False), (2048, 2048, 2, 128, True)]
+    ws = []
+    for i, (k, n, q, g, off) in enumerate(shapes):
+        w, W = make(lutgemm, synth, k, n, q, g, offset=off, seed=50 + i)
+        W.set_plan(4, 2)
+        ws.append((w, W))
+    clones = [ws[0][1].clone() for _ in range(40)]          # forty more independent copies of shape 0
+    xh = {k: synth.make_x(2, k, seed=k) for k in (2048, 4096)}
+    xs = {k: torch.from_numpy(v).to(device) for k, v in xh.items()}
+
+    def buf(n, m=1):
+        return torch.full((m, n), float("nan"), dtype=torch.float16, device=device)
+
+    entries = []            # (weight, x tensor, y tensor, m, synthetic weight or None, host x, exact?)
+    for c in clones:                                            # 40 equal shapes: launches of 32 + 8 and more
+        entries.append((c, xs[2048][0], buf(2048), 1, ws[0][0], xh[2048][0:1], False))
+    entries.append((ws[1][1], xs[2048][0], buf(1000), 1, ws[1][0], xh[2048][0:1], False))   # other n: joins the run
+    entries.append((ws[2][1], xs[4096][0], buf(2048), 1, ws[2][0], xh[4096][0:1], False))   # other k, g = 256: joins
+    entries.append((ws[3][1], xs[2048][1], buf(2048), 1, ws[3][0], xh[2048][1:2], True))    # g = 64: another kernel, alone
+    entries.append((ws[4][1], xs[2048][1], buf(2048), 1, ws[4][0], xh[2048][1:2], True))    # q = 2 with offset: alone
+    entries.append((ws[0][1], xs[2048][0], buf(2048), 1, ws[0][0], xh[2048][0:1], True))
+    entries.append((ws[0][1], xs[2048][1], buf(2048), 1, ws[0][0], xh[2048][1:2], True))    # same handle twice in a row
+    entries.append((ws[1][1], xs[2048], buf(1000, 2), 2, ws[1][0], xh[2048], True))         # two rows
+    chain_in = buf(2048)
+    entries.append((ws[0][1], xs[2048][0], chain_in, 1, ws[0][0], xh[2048][0:1], True))
+    entries.append((clones[0], chain_in[0], buf(2048), 1, None, None, True))               # reads the previous output
+    want = []
+    for W, x, y, m, _, _, _ in entries:
+        ref = torch.full_like(y, float("nan"))
+        W.matvec(x.data_ptr(), ref.data_ptr(), m, st)
+        torch.cuda.synchronize()
+        if y is chain_in:
+            chain_in.copy_(ref)       # the next reference call reads it
+        want.append(ref)
+    chain_in.fill_(float("nan"))
+    seq = lutgemm.MatvecSequence([(e[0], e[1].data_ptr(), e[2].data_ptr(), e[3]) for e in entries])
+    first = None
+    for rep in range(3):
+        for e in entries:
+            e[2].fill_(float("nan"))
+        seq.launch(st)
+        torch.cuda.synchronize()
+        got = [e[2].clone() for e in entries]
+        for idx, (e, ref, y) in enumerate(zip(entries, want, got)):
+            if e[6]:
+                assert torch.equal(y.view(torch.int16), ref.view(torch.int16)), "entry %d, repetition %d" % (idx, rep)
+            if e[4] is not None and rep == 0:
+                assert_within_tolerance(y.cpu().numpy(), truth_of(oracle, e[4], e[5]), "entry %d" % idx)
+        if first is None:
+            first = got
+        else:
+            assert all(torch.equal(a.view(torch.int16), b.view(torch.int16)) for a, b in zip(first, got)), rep
+    for c in clones:
+        c.close()
+    for _, W in ws:
+        W.close()
+
+
 def test_one_handle_on_two_streams(lutgemm, oracle, device):
     """Every stream that launches on a handle has split-k words of its own: launches that
     overlap on two streams give the results of the same launches issued one after the other."""
