@@ -38,11 +38,11 @@ for _p in (ROOT, os.path.join(ROOT, "lut-gemm_amd")):
 HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published peak
 LLC_BYTES = 256 << 20  # last-level (memory-side) cache
 METRIC = "µs/matvec + weight-GB/s (% HBM peak), n=k=12288 q=3 g=128 m=1 fp16"
-# HBM bytes per cfg1 launch from the rocprofv3 counter runs summarised in
-# profiles/lut_matvec_kernel_cfg1.md (FETCH_SIZE and WRITE_SIZE, scaled by the factors a plain
-# copy kernel of known size reads on the same counters)
-# (64.01 MB read for either plan; 0.91 MB written with 8 k-splits, 0.61 MB with 5: fewer split-k atomics)
-CFG1_MEASURED_TRAFFIC_BYTES_PER_MATVEC = None  # set from the counter runs of the fused kernel (profiles/)
+# HBM bytes per cfg1 matvec inside a launch of lutgemm_matvec_many, from the rocprofv3 counter runs
+# summarised in profiles/lut_matvec_multi_kernel_cfg1.md (FETCH_SIZE and WRITE_SIZE per dispatch,
+# scaled by the factors a plain copy kernel of known size reads on the same counters, divided by
+# the matvecs of the dispatch): 63.72 MB read + 0.32 MB written
+CFG1_MEASURED_TRAFFIC_BYTES_PER_MATVEC = 64.04e6
 
 
 def event_time_ms(torch, fn, stream):
