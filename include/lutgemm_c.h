@@ -85,11 +85,17 @@ int lutgemm_weight_info(const lutgemm_weight *w, lutgemm_weight_info_t *info);
  * call allocates nothing.  The result is deterministic (bit-identical from launch to launch).
  * Replaces lutGEMM::matmul(void* output, void* input, nQWeight_fp16&, int m, int algo)
  * (lutGEMM/include/kernels.h:27, lutGEMM/src/kernels.cu:64-71), which for m == 1 runs
- * kernel::nqmv (mv_fp16.hpp:121) or kernel::nqmv_bias (mv_fp16_bias.hpp:143); here every
- * 1 <= m <= LUTGEMM_MAX_BATCH stays on the table-lookup kernels: rows go through the weight two
- * per pass (one for a last odd row), every row bit-identical to its own one-row call.
+ * kernel::nqmv (mv_fp16.hpp:121) or kernel::nqmv_bias (mv_fp16_bias.hpp:143) and for m > 1
+ * dequantises the whole weight and calls a library GEMM (kernels.cu:73-79); here every
+ * 1 <= m <= LUTGEMM_MAX_BATCH streams the packed weight: m == 1 and m == 2 through the table-lookup
+ * kernels (a two-row pass gives each row bit-identical to its own one-row call), m >= 3 through
+ * the batch kernel, which takes up to 16 rows per pass over the weight and contracts them on the
+ * matrix cores while a tile is in registers (group sizes that are multiples of 128; other group
+ * sizes take table-lookup passes of two rows).  Batch results are deterministic and within the
+ * same tolerance, but a row may differ in the last bit from its own one-row call (another order
+ * of the fp32 additions).
  * Launches on one stream run one after the other and share the handle's split-k accumulators;
- * every further stream that launches on the handle gets accumulators of its own (eight streams
+ * every further stream that launches on the handle gets accumulators of its own (four streams
  * per handle, LUTGEMM_ERR_UNSUPPORTED beyond; lutgemm_weight_reset_workspace releases them), so
  * launches on different streams may overlap in time.  Launches from different host threads on the
  * SAME stream must be serialised by the caller, as for any stream.
@@ -117,7 +123,7 @@ int lutgemm_matvec_static(const lutgemm_weight *w, const void *x, void *y, int m
  * Replaces lutGEMM::matmul(void* output, nQWeight_fp16&, void* input, int n, int algo)
  * (lutGEMM/include/kernels.h:26, lutGEMM/src/kernels.cu:56-63).  For m == 1 it is the same
  * operation as lutgemm_matvec.  For m > 1 the columns are first gathered into a staging buffer
- * owned by the handle (one per launching stream).  Up to m = 8 nothing is allocated; a larger m
+ * owned by the handle (one per launching stream).  Up to m = 16 nothing is allocated; a larger m
  * grows the buffer the first time it occurs (device synchronisation, free and allocation). */
 int lutgemm_matvec_cols(const lutgemm_weight *w, const void *x, void *y, int m, void *stream);
 

@@ -1,0 +1,376 @@
+// gfx950 kernel for small batches: 3..16 activation rows against a packed BCQ weight in ONE pass
+// over its tiles.
+//
+// The reference sends every batch larger than one row through a dense round trip: it dequantises
+// the whole weight to fp16 in a scratch buffer and calls a library GEMM
+// (lutGEMM/src/kernels.cu:73-79, lutGEMM/src/nQWeight_fp16.cu:93-99).  Here the packed tiles are
+// streamed once, exactly as the one-row kernel streams them, and the batch is contracted on the
+// matrix cores while the tile is in registers:
+//
+//  * A sign byte (8 consecutive k of one output, one plane) is the B operand of one lane of a
+//    v_mfma_f32_16x16x32_f16: its 8 sign bits become 8 fp16 values +1 / -1 by a 16-byte read from
+//    a constant table in LDS (256 patterns, replicated per lane slot so that the reads are
+//    bank-conflict free).  MFMA lane (kappa = lane / 16, j = lane % 16) supplies output j and, in
+//    MFMA t of a k-block, chunk 4 t + kappa: the four k groups of an MFMA are four neighbouring
+//    chunks, so an MFMA never mixes two scale groups and four MFMAs cover one 128-k group.
+//  * The tiles arrive "k across lanes" (lane = chunk, 16 bytes = 16 outputs).  Per 16-byte sign
+//    vector the wavefront transposes 4 x 4 byte blocks among the lanes c, c+4, c+8, c+12 of a row
+//    (DPP moves and byte permutes), writes four dwords into a 1 KiB staging area in LDS laid out
+//    [output][chunk position (c % 4) * 16 + c / 4] and reads 16 bytes back: lane (kappa, j) then
+//    holds the sign bytes of output j for chunks kappa, kappa + 4, ..., kappa + 60 in MFMA order.
+//  * The A operand is the activation block: lane (kappa, i) holds x[row i][8 k of chunk
+//    4 t + kappa], read from an LDS copy that the workgroup shares (rows beyond the batch are zero).
+//  * After the four MFMAs of a group, the 16 x 16 result (rows x outputs) is multiplied by the
+//    fp16 scale of that (plane, group, output) and added to the fp32 accumulators; the offset
+//    term uses the group sums of x, which one more MFMA chain with an all-ones operand provides.
+//    Products of fp16 numbers are exact in fp32, so the only roundings are fp32 additions.
+//  * At the end every (row, output) goes through the same split-k completion as the one-row kernel.
+//
+// Only scale layouts with one group per 128 k (group size a multiple of 128) are handled here;
+// other group sizes keep the two-row table kernel.
+#include <hip/hip_fp16.h>
+#include <hip/hip_runtime.h>
+
+#include <atomic>
+
+#include "device_util.h"
+#include "kernels.h"
+#include "layout.h"
+#include "tile_device.h"
+
+namespace lutgemm_kernels {
+using namespace lutgemm_layout;
+
+namespace {
+
+typedef _Float16 half8 __attribute__((ext_vector_type(8)));
+typedef float float4v __attribute__((ext_vector_type(4)));
+typedef __attribute__((address_space(3))) unsigned char lds_byte;
+
+constexpr int kPatternBytes = 256 * 16 * 16;               // 64 KiB: [pattern][lane slot][16 bytes]
+constexpr int kXRowBytes = kBlockK * 2 + 16;               // one activation row of a k-block, padded:
+                                                           // 16 rows read at one column hit 64 different banks
+constexpr int kXBufBytes = kBatchRows * kXRowBytes;        // 16,640
+constexpr int kStageBytes = 1024;                          // per wavefront: [16 outputs][64 chunk positions]
+constexpr int kBatchMaxWaves = 8;                          // the kernel is compiled for at most 512 threads
+
+__host__ __device__ constexpr int batch_lds_bytes(int waves)
+{
+    return kPatternBytes + 2 * kXBufBytes + waves * kStageBytes;
+}
+
+// 4 x 4 byte transpose among the lanes c, c + 4, c + 8, c + 12 of a 16-lane row: the lane with
+// e = (lane / 4) % 4 ends with byte e of the dwords of those four lanes, in lane order.
+__device__ __forceinline__ uint32_t stride4_transpose(uint32_t v, uint32_t sel1, uint32_t sel2)
+{
+    // partner lane ^ 4: lanes 0-3 and 8-11 of a row fetch from lane + 4, the others from lane - 4
+    const uint32_t p1 = (uint32_t)__builtin_amdgcn_update_dpp(
+        __builtin_amdgcn_update_dpp(0, (int)v, 0x104 /* row_shl:4 */, 0xf, 0x5, false), (int)v, 0x114 /* row_shr:4 */,
+        0xf, 0xa, false);
+    const uint32_t a = __builtin_amdgcn_perm(p1, v, sel1);
+    // partner lane ^ 8: rotate the row by 8
+    const uint32_t p2 = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)a, 0x128 /* row_ror:8 */, 0xf, 0xf, false);
+    return __builtin_amdgcn_perm(p2, a, sel2);
+}
+
+// The activation block of k-block ts is 16 rows x 64 chunks = 1024 pieces of 16 bytes; thread tid
+// moves pieces tid and tid + threads (workgroups have exactly 8 wavefronts).
+// Loads and LDS writes are separate so that the loads of the next block are in flight while the
+// current one is processed.  Rows beyond the batch and k beyond the weight are zero.
+constexpr int kMaxPieces = 2;
+struct ActivationPieces {
+    u32x4 v[kMaxPieces];
+};
+
+__device__ __forceinline__ void load_activation_pieces(ActivationPieces &p, const MatvecArgs &a, int ts, int tid,
+                                                       int threads, bool valid)
+{
+    // Branch free (a masked address and masked data instead of a conditional load), so that the
+    // compiler's wait counts for the loads around it stay exact.
+    const __half *x = reinterpret_cast<const __half *>(a.x);
+#pragma unroll
+    for (int i = 0; i < kMaxPieces; i++) {
+        const int piece = (tid + i * threads) & (kBatchRows * kLanes - 1);
+        const int r = piece >> 6, c = piece & 63;
+        const int kpos = ts * kBlockK + c * kChunk;
+        const uint32_t m = 0u - (uint32_t)(valid && r < a.rows && kpos < a.k);
+        const size_t offset = ((size_t)r * (size_t)a.x_row_stride + (size_t)kpos) & (size_t)(0 - (long long)(m & 1u));
+        u32x4 v = *reinterpret_cast<const u32x4 *>(x + offset);
+        v.x &= m;
+        v.y &= m;
+        v.z &= m;
+        v.w &= m;
+        p.v[i] = v;
+    }
+}
+
+__device__ __forceinline__ void store_activation_pieces(const ActivationPieces &p, lds_byte *buf, int tid, int threads)
+{
+#pragma unroll
+    for (int i = 0; i < kMaxPieces; i++) {
+        const int piece = tid + i * threads;
+        const int r = piece >> 6, c = piece & 63;
+        if (piece < kBatchRows * kLanes)
+            *reinterpret_cast<__attribute__((address_space(3))) u32x4 *>(buf + r * kXRowBytes + c * 16) = p.v[i];
+    }
+}
+
+template <int Q, bool OFF>
+__global__ __launch_bounds__(512) void lut_batch_kernel(MatvecArgs a)
+{
+    constexpr int QO = Q + (OFF ? 1 : 0);
+    constexpr int NU = 2 * Q;   // sign vectors (units) of a tile: unit U = plane U / 2, output half U % 2
+    constexpr int CH = NU <= 6 ? NU : NU % 6 == 0 ? 6 : NU % 5 == 0 ? 5 : NU % 4 == 0 ? 4 : 2;   // units per pass
+    // The kernel's only LDS object, so it starts at LDS address 0: pattern addresses are formed
+    // from the sign byte and a lane constant alone.
+    extern __shared__ __attribute__((aligned(16))) unsigned char lds_generic[];
+    lds_byte *lds = (lds_byte *)lds_generic;
+    lds_byte *pattern = lds;
+    lds_byte *xbuf = lds + kPatternBytes;
+
+    const int tid = threadIdx.x;
+    const int threads = blockDim.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int waves = threads >> 6;
+    const int ntile = blockIdx.x % a.ntiles;
+    const int ks = blockIdx.x / a.ntiles;
+    const int nb = ntile * waves + wave;
+    const bool active = nb < a.nb;
+    const int ts0 = ks * a.blocks_per_split;
+    const int ts1 = min(ts0 + a.blocks_per_split, a.ts);
+    lds_byte *stage = lds + kPatternBytes + 2 * kXBufBytes + wave * kStageBytes;
+
+    // Sign patterns: entry e, dword v holds the fp16 pair for bits 2v and 2v+1 of e: +1.0 where
+    // the bit is set, -1.0 where it is clear.  All 16 lane slots of an entry hold the same 16 bytes.
+    for (int idx = tid; idx < 256 * 16; idx += threads) {
+        const uint32_t e = (uint32_t)idx >> 4;
+        u32x4 m;
+        m.x = (((e >> 0) & 1u) ? 0x3c00u : 0xbc00u) | (((e >> 1) & 1u) ? 0x3c000000u : 0xbc000000u);
+        m.y = (((e >> 2) & 1u) ? 0x3c00u : 0xbc00u) | (((e >> 3) & 1u) ? 0x3c000000u : 0xbc000000u);
+        m.z = (((e >> 4) & 1u) ? 0x3c00u : 0xbc00u) | (((e >> 5) & 1u) ? 0x3c000000u : 0xbc000000u);
+        m.w = (((e >> 6) & 1u) ? 0x3c00u : 0xbc00u) | (((e >> 7) & 1u) ? 0x3c000000u : 0xbc000000u);
+        *reinterpret_cast<__attribute__((address_space(3))) u32x4 *>(pattern + idx * 16) = m;
+    }
+    ActivationPieces pieces;
+    load_activation_pieces(pieces, a, ts0, tid, threads, true);
+    store_activation_pieces(pieces, xbuf, tid, threads);
+
+    const u32x4 *signs = reinterpret_cast<const u32x4 *>(a.signs);
+    const uint32_t *scales = reinterpret_cast<const uint32_t *>(a.scales);
+    const size_t tile0 = (size_t)(active ? nb : 0) * a.ts;
+
+    // lane roles
+    const int kappa = lane >> 4, j = lane & 15;       // MFMA: k group and output column / activation row
+    const uint32_t sel1 = (lane & 4) ? 0x03070105u : 0x06020400u;
+    const uint32_t sel2 = (lane & 8) ? 0x03020706u : 0x05040100u;
+    // staging: lane (row r, e = (lane / 4) % 4, e0 = lane % 4) writes dword d of a unit to
+    // [output 4 d + e][positions e0 * 16 + 4 r .. + 3]
+    __attribute__((address_space(3))) uint32_t *stage_w = reinterpret_cast<__attribute__((address_space(3))) uint32_t *>(
+        stage + ((lane >> 2) & 3) * 64 + (lane & 3) * 16 + (lane >> 4) * 4);
+    const __attribute__((address_space(3))) u32x4 *stage_r =
+        reinterpret_cast<const __attribute__((address_space(3))) u32x4 *>(stage + j * 64 + kappa * 16);
+    // bytes 0, 2 and 3 of a pattern address: lane slot and the LDS address bits above 64 KiB
+    const uint32_t pattern_lane = ((uint32_t)j << 4) + (uint32_t)(size_t)pattern;
+
+    // The sign vectors of a tile as in the one-row kernel.  Scale words: those of ALL four 128-k
+    // groups of the k-block for this lane's two outputs (j and 16 + j); group r is held by lane
+    // 16 r + j of the scale tile.  Both are fetched one k-block ahead.
+    u32x4 sign[NU];
+    uint32_t sc[4][QO];
+    auto scale_address = [&](size_t tile, int r, bool real) {
+        const size_t m = (size_t)0 - (size_t)real;
+        return scales + (((tile * kLanes + 16 * r + j) * (size_t)QO) & m);
+    };
+    {
+        const NextTile n0 = tile_address<Q, QO, 1>(signs, scales, tile0 + ts0, lane, true);
+#pragma unroll
+        for (int r = 0; r < 4; r++)
+#pragma unroll
+            for (int d = 0; d < QO; d++) sc[r][d] = __builtin_nontemporal_load(scale_address(tile0 + ts0, r, true) + d);
+#pragma unroll
+        for (int u = 0; u < NU; u++) sign[u] = __builtin_nontemporal_load(n0.sign + u * n0.sign_stride);
+    }
+
+    float4v acc[2];
+    acc[0] = float4v{0.f, 0.f, 0.f, 0.f};
+    acc[1] = float4v{0.f, 0.f, 0.f, 0.f};
+    const float4v zero4 = float4v{0.f, 0.f, 0.f, 0.f};
+    const u32x4 ones = {0x3c003c00u, 0x3c003c00u, 0x3c003c00u, 0x3c003c00u};
+
+    __syncthreads();
+    for (int ts = ts0; ts < ts1; ts++) {
+        const int cur = (ts - ts0) & 1;
+        const bool more = ts + 1 < ts1;
+        const NextTile next = tile_address<Q, QO, 1>(signs, scales, tile0 + ts + 1, lane, more);
+        load_activation_pieces(pieces, a, ts + 1, tid, threads, more);
+
+        // scale words of this k-block (two fp16 per word), then the refill of their registers
+        uint32_t scw[4][QO];
+#pragma unroll
+        for (int r = 0; r < 4; r++)
+#pragma unroll
+            for (int d = 0; d < QO; d++) scw[r][d] = sc[r][d];
+#pragma unroll
+        for (int r = 0; r < 4; r++)
+#pragma unroll
+            for (int d = 0; d < QO; d++) sc[r][d] = __builtin_nontemporal_load(scale_address(tile0 + ts + 1, r, more) + d);
+        // fp16 number hb (= output half * QO + plane-or-offset) of group r as fp32
+        auto scale_of = [&](int r, int hb) {
+            const __half2 h2 = *reinterpret_cast<const __half2 *>(&scw[r][hb >> 1]);
+            return (hb & 1) ? __high2float(h2) : __low2float(h2);
+        };
+
+        const lds_byte *xr = xbuf + cur * kXBufBytes + j * kXRowBytes + kappa * 16;
+        // The sign vectors are taken CH at a time (all of them up to three planes), so that the
+        // registers of a pass stay within the budget for any number of planes.
+        static_for<NU / CH>([&](auto C) {
+            constexpr int u0 = C * CH;
+            // transpose; the registers of a sign vector are refilled right away
+            u32x4 R[CH];
+            static_for<CH>([&](auto I) {
+                constexpr int U = u0 + I;
+                const u32x4 w4 = sign[U];
+                stage_w[0 * 64] = stride4_transpose(w4.x, sel1, sel2);
+                stage_w[1 * 64] = stride4_transpose(w4.y, sel1, sel2);
+                stage_w[2 * 64] = stride4_transpose(w4.z, sel1, sel2);
+                stage_w[3 * 64] = stride4_transpose(w4.w, sel1, sel2);
+                R[I] = *stage_r;
+                sign[U] = __builtin_nontemporal_load(next.sign + U * next.sign_stride);
+            });
+            static_for<4>([&](auto G) {   // the four 128-k groups of the k-block
+                constexpr int r = G;
+                float4v part[CH];
+                float4v xsum = zero4;
+                static_for<4>([&](auto TT) {
+                    constexpr int t = 4 * r + TT;   // MFMA t: chunks 4 t .. 4 t + 3
+                    const half8 xa = *reinterpret_cast<const __attribute__((address_space(3))) half8 *>(xr + t * 64);
+                    static_for<CH>([&](auto I) {
+                        constexpr uint32_t sel = 0x03020400u + ((uint32_t)(t & 3) << 8);   // address byte 1 <- sign byte t % 4
+                        const uint32_t word = t < 4 ? R[I].x : t < 8 ? R[I].y : t < 12 ? R[I].z : R[I].w;
+                        const uint32_t addr = __builtin_amdgcn_perm(word, pattern_lane, sel);
+                        const half8 bits = *reinterpret_cast<const __attribute__((address_space(3))) half8 *>(addr);
+                        part[I] = __builtin_amdgcn_mfma_f32_16x16x32_f16(xa, bits, TT == 0 ? zero4 : part[I], 0, 0, 0);
+                    });
+                    if constexpr (OFF && C == 0 && NU <= 6)
+                        xsum = __builtin_amdgcn_mfma_f32_16x16x32_f16(xa, __builtin_bit_cast(half8, ones), xsum, 0, 0, 0);
+                });
+                static_for<CH>([&](auto I) {
+                    constexpr int U = u0 + I, b = U / 2, h = U % 2;
+                    const float s = scale_of(r, h * QO + b);
+                    acc[h][0] += s * part[I][0];
+                    acc[h][1] += s * part[I][1];
+                    acc[h][2] += s * part[I][2];
+                    acc[h][3] += s * part[I][3];
+                });
+                if constexpr (OFF && C == 0 && NU <= 6) {
+#pragma unroll
+                    for (int h = 0; h < 2; h++) {
+                        const float z = scale_of(r, h * QO + Q);
+                        acc[h][0] += z * xsum[0];
+                        acc[h][1] += z * xsum[1];
+                        acc[h][2] += z * xsum[2];
+                        acc[h][3] += z * xsum[3];
+                    }
+                }
+                if constexpr (NU > 6) __builtin_amdgcn_sched_barrier(0);   // many planes: keep the groups' registers apart
+            });
+            __builtin_amdgcn_sched_barrier(0);   // one pass after the other: keeps the registers of a pass apart
+        });
+        if constexpr (OFF && NU > 6) {   // many planes: the offset term in a pass of its own
+            static_for<4>([&](auto G) {
+                constexpr int r = G;
+                float4v xsum = zero4;
+                static_for<4>([&](auto TT) {
+                    constexpr int t = 4 * r + TT;
+                    const half8 xa = *reinterpret_cast<const __attribute__((address_space(3))) half8 *>(xr + t * 64);
+                    xsum = __builtin_amdgcn_mfma_f32_16x16x32_f16(xa, __builtin_bit_cast(half8, ones), xsum, 0, 0, 0);
+                });
+#pragma unroll
+                for (int h = 0; h < 2; h++) {
+                    const float z = scale_of(r, h * QO + Q);
+                    acc[h][0] += z * xsum[0];
+                    acc[h][1] += z * xsum[1];
+                    acc[h][2] += z * xsum[2];
+                    acc[h][3] += z * xsum[3];
+                }
+            });
+        }
+        store_activation_pieces(pieces, xbuf + (cur ^ 1) * kXBufBytes, tid, threads);
+        __syncthreads();   // the next activation block is in place; this one is no longer read
+    }
+
+    // acc[h][v]: activation row 4 kappa + v, output nb * 32 + 16 h + j.  All eight split-k atomics
+    // of a lane are issued before the first answer is looked at.
+    __half *y = reinterpret_cast<__half *>(a.y);
+    bool valid[2][4];
+    unsigned long long *word[2][4];
+    __half *yout[2][4];
+#pragma unroll
+    for (int h = 0; h < 2; h++)
+#pragma unroll
+        for (int v = 0; v < 4; v++) {
+            const int row = 4 * kappa + v, out = nb * kBatch + 16 * h + j;
+            valid[h][v] = active && row < a.rows && out < a.n;
+            word[h][v] = a.accum + (size_t)row * a.accum_row_stride + out;
+            yout[h][v] = y + (size_t)row * a.y_row_stride + (size_t)out * a.y_stride;
+        }
+    if (a.k_splits == 1) {
+#pragma unroll
+        for (int h = 0; h < 2; h++)
+#pragma unroll
+            for (int v = 0; v < 4; v++)
+                if (valid[h][v]) *yout[h][v] = __float2half_rn(acc[h][v]);
+        return;
+    }
+    Arrival arrival[2][4];
+#pragma unroll
+    for (int h = 0; h < 2; h++)
+#pragma unroll
+        for (int v = 0; v < 4; v++) arrival[h][v] = arrive_output(acc[h][v], valid[h][v], word[h][v]);
+#pragma unroll
+    for (int h = 0; h < 2; h++)
+#pragma unroll
+        for (int v = 0; v < 4; v++) complete_output(arrival[h][v], valid[h][v], word[h][v], yout[h][v], a.k_splits);
+}
+
+template <int Q, bool OFF>
+hipError_t launch_batch_q(const MatvecArgs &a, int workgroups, int waves, hipStream_t stream)
+{
+    static std::atomic<unsigned long long> allowed{0};
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return e;
+    const unsigned long long bit = 1ull << (dev & 63);
+    if (!(allowed.load(std::memory_order_relaxed) & bit)) {
+        e = hipFuncSetAttribute(reinterpret_cast<const void *>(&lut_batch_kernel<Q, OFF>),
+                                hipFuncAttributeMaxDynamicSharedMemorySize, batch_lds_bytes(kBatchMaxWaves));
+        if (e != hipSuccess) return e;
+        allowed.fetch_or(bit, std::memory_order_relaxed);
+    }
+    hipLaunchKernelGGL((lut_batch_kernel<Q, OFF>), dim3(workgroups), dim3(waves * kLanes), batch_lds_bytes(waves), stream,
+                       a);
+    return hipGetLastError();
+}
+
+template <int Q>
+hipError_t launch_batch_off(int has_offset, const MatvecArgs &a, int wg, int waves, hipStream_t s)
+{
+    return has_offset ? launch_batch_q<Q, true>(a, wg, waves, s) : launch_batch_q<Q, false>(a, wg, waves, s);
+}
+
+}  // namespace
+
+hipError_t launch_batch(int q, int has_offset, const MatvecArgs &a, int workgroups, int waves, hipStream_t stream)
+{
+    if (a.rows < 1 || a.rows > kBatchRows || waves != kBatchMaxWaves) return hipErrorInvalidValue;
+    switch (q) {
+        case 1: return launch_batch_off<1>(has_offset, a, workgroups, waves, stream);
+        case 2: return launch_batch_off<2>(has_offset, a, workgroups, waves, stream);
+        case 3: return launch_batch_off<3>(has_offset, a, workgroups, waves, stream);
+        case 4: return launch_batch_off<4>(has_offset, a, workgroups, waves, stream);
+        default: return hipErrorInvalidValue;   // more planes than kBatchMaxPlanes
+    }
+}
+
+}  // namespace lutgemm_kernels

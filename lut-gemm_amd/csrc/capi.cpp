@@ -43,9 +43,10 @@ int hip_fail(hipError_t e, const char *what)
 constexpr int kMaxWaves = 12;  // the kernel is compiled for at most 768 threads per workgroup
 constexpr int kBuildRounds = 8;  // table parts per k-block (kernels.hip: kBuildParts)
 constexpr int kMaxSplits = 128;  // the split-k arrival count has 8 bits, the sum room for 128 addends
-constexpr int kStreamSlots = 8;  // sets of split-k words per handle: one per stream that launches on it
-constexpr int kRowsPerPass = 2;  // activation rows a launch can take (rows of split-k words per slot)
-constexpr int kStagedColumns = 8;  // column-batched calls up to this m never allocate
+constexpr int kStreamSlots = 4;  // sets of split-k words per handle: one per stream that launches on it
+constexpr int kRowsPerPass = lutgemm_kernels::kBatchRows;  // activation rows a launch can take (rows of split-k words per set)
+constexpr int kTableRows = 2;    // rows per pass of the table-lookup kernels
+constexpr int kStagedColumns = 16;  // column-batched calls up to this m never allocate
 
 struct Plan {
     int waves;             // wavefronts (= output batches) per workgroup
@@ -174,6 +175,33 @@ FusedPlan choose_fused_plan(const Shape *const *shapes, int count, int cus)
                 best = FusedPlan{waves, bpg};
             }
         }
+    return best;
+}
+
+// Launch plan of the batch kernel (3..16 rows per pass on the matrix cores): 8 wavefronts per
+// workgroup; the k-split is chosen so that the rounds of workgroups are full.  Per k-block a
+// workgroup is bound by its LDS reads (16 bytes per lane and sign byte for the matrix operand:
+// 32 q + 16 + 2 q reads of 1 KiB per tile at 128 bytes per clock), not by the stream; start and
+// end of a workgroup (pattern table, first activation block, split-k atomics) cost about 3 us.
+Plan choose_batch_plan(const Shape &s, int cus)
+{
+    const int waves = 8;
+    const int ntiles = div_up(s.nb, waves);
+    const double kClockMHz = 2300.0, kStartEnd = 3.0, kBytesPerCu = 7.0e6 / 256.0;
+    const double t_lds = 1.2 * waves * (34.0 * s.q + 16.0) * 8.0 / kClockMHz;
+    const double t_mem = waves * (double)(sign_tile_bytes(s) + scale_tile_bytes(s)) / kBytesPerCu;
+    const double t_block = t_lds > t_mem ? t_lds : t_mem;
+    Plan best{waves, ntiles, s.ts, 1};
+    double best_cost = 1e300;
+    for (int bps = div_up(s.ts, kMaxSplits); bps <= s.ts; bps++) {
+        const int ks = div_up(s.ts, bps);
+        const long groups = (long)ntiles * ks;
+        const double cost = (double)((groups + cus - 1) / cus) * (bps * t_block + kStartEnd);
+        if (cost < best_cost - 1e-9) {
+            best_cost = cost;
+            best = Plan{waves, ntiles, bps, ks};
+        }
+    }
     return best;
 }
 
@@ -422,10 +450,10 @@ int run_matvec(const lutgemm_weight *w, const void *x, void *y, int m, void *str
     int slot = 0;
     if (static_ws) {
         const size_t words = lutgemm_kernels::kStaticSplitKWords;
-        if ((size_t)kRowsPerPass * s.nb * kBatch > words)
+        if ((size_t)kTableRows * s.nb * kBatch > words)
             return fail(LUTGEMM_ERR_UNSUPPORTED,
                         "n=%d is beyond what the static workspace holds (%zu outputs per activation row)", s.n,
-                        words / kRowsPerPass);
+                        words / kTableRows);
         hipError_t es = lutgemm_kernels::static_split_k_words(w->device, &a.accum);
         if (es != hipSuccess) return hip_fail(es, "hipGetSymbolAddress(static split-k words)");
         if (g_static_dirty[w->device]) {  // a launch failed half way through a call: start from zero again
@@ -455,9 +483,32 @@ int run_matvec(const lutgemm_weight *w, const void *x, void *y, int m, void *str
         if (e != hipSuccess) return hip_fail(e, "launch gather_columns_kernel");
         xh = rows;
     }
-    // two activation rows per pass over the weight, a last single row if m is odd
     a.x_row_stride = s.k;
     a.accum_row_stride = (long long)s.nb * kBatch;
+    if (m >= 3 && s.gsub == 1 && s.q <= lutgemm_kernels::kBatchMaxPlanes && !static_ws) {
+        // up to 16 rows per pass over the weight on the matrix cores
+        const Plan plan = choose_batch_plan(s, w->compute_units);
+        a.ntiles = plan.ntiles;
+        a.k_splits = plan.k_splits;
+        a.blocks_per_split = plan.blocks_per_split;
+        for (int r = 0; r < m; r += kRowsPerPass) {
+            a.rows = m - r < kRowsPerPass ? m - r : kRowsPerPass;
+            a.x = xh + (size_t)r * s.k;
+            if (cols) {  // y [n][m]
+                a.y = yh + r;
+                a.y_stride = m;
+                a.y_row_stride = 1;
+            } else {     // y [m][n]
+                a.y = yh + (size_t)r * s.n;
+                a.y_stride = 1;
+                a.y_row_stride = s.n;
+            }
+            hipError_t e = lutgemm_kernels::launch_batch(s.q, s.has_offset, a, plan.ntiles * plan.k_splits, plan.waves, st);
+            if (e != hipSuccess) return hip_fail(e, "launch lut_batch_kernel");
+        }
+        return LUTGEMM_OK;
+    }
+    // two activation rows per pass over the weight, a last single row if m is odd
     for (int r = 0; r < m; r += 2) {
         a.rows = m - r >= 2 ? 2 : 1;
         const Plan &plan = a.rows == 2 ? w->plan2 : w->plan;

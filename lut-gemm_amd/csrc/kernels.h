@@ -23,9 +23,13 @@ struct MatvecArgs {
     int y_stride;           // output j goes to y[j * y_stride]
     // rows == 2: a second activation row at x + x_row_stride goes to y + y_row_stride in the
     // same pass (strides in fp16 elements), with its accumulators at accum + accum_row_stride
-    int rows;               // 1 or 2 activation rows (0 selects the read probe)
+    int rows;               // 1 or 2 activation rows (0 selects the read probe); 1..kBatchRows for launch_batch
     long long x_row_stride, y_row_stride, accum_row_stride;
 };
+
+// Activation rows the batch kernel takes in one pass over the weight (rows r at x + r * x_row_stride
+// go to y + r * y_row_stride, with split-k accumulators at accum + r * accum_row_stride).
+constexpr int kBatchRows = 16;
 
 // Up to kMaxFused independent one-row matvecs for one launch: entry i owns the workgroups
 // first_block[i] .. first_block[i+1]-1 of the grid (the last entry up to the end).
@@ -51,6 +55,11 @@ hipError_t launch_matvec(int q, int has_offset, int gsub, const MatvecArgs &a, i
 // entries with rows == 1 sharing q, has_offset, gsub and the wavefronts per workgroup
 hipError_t launch_matvec_multi(int q, int has_offset, int gsub, const MultiMatvecArgs &m, int workgroups, int waves,
                                hipStream_t stream);
+
+// 1..kBatchRows activation rows in one pass (matrix cores); scale layouts with gsub == 1 and up to
+// kBatchMaxPlanes planes only, exactly 8 wavefronts per workgroup.
+constexpr int kBatchMaxPlanes = 4;
+hipError_t launch_batch(int q, int has_offset, const MatvecArgs &a, int workgroups, int waves, hipStream_t stream);
 
 // words[0..count) = 0 (a fill kernel rather than a memset node, so that it can be captured)
 hipError_t launch_fill_zero(unsigned long long *words, size_t count, hipStream_t stream);

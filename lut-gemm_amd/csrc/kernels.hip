@@ -31,6 +31,7 @@
 #include "device_util.h"
 #include "kernels.h"
 #include "layout.h"
+#include "tile_device.h"
 
 namespace lutgemm_kernels {
 using namespace lutgemm_layout;
@@ -307,45 +308,6 @@ __device__ __forceinline__ void build_part2(float2 *col, int part, const float (
 }
 
 
-template <int Q, int QO, int GSUB>
-struct TileRegs {
-    u32x4 sign[2 * Q];
-    uint32_t scale[GSUB * QO];
-};
-
-// Where the next tile's loads of a wavefront come from (all lanes the same dummy line when the
-// workgroup has no next k-block, see tile_address).
-struct NextTile {
-    const u32x4 *sign;    // this lane's first sign vector
-    size_t sign_stride;   // in u32x4 units between units
-    const uint32_t *scale;
-};
-
-// Addresses of tile `tile` for this lane.  `real` is wave-uniform; when false every lane reads
-// the first bytes of the arrays instead (one cached line).  Written with masks rather than
-// conditionals so that no branch appears: with straight-line code the compiler's wait counts
-// for the loads stay exact.
-template <int Q, int QO, int GSUB>
-__device__ __forceinline__ NextTile tile_address(const u32x4 *signs, const uint32_t *scales, size_t tile,
-                                                 int lane, bool real)
-{
-    const size_t m = (size_t)0 - (size_t)real;  // all ones or zero
-    NextTile n;
-    n.scale = scales + (((tile * kLanes + lane) * (size_t)(GSUB * QO)) & m);
-    n.sign = signs + ((tile * (size_t)(2 * Q * kLanes) + lane) & m);
-    n.sign_stride = (size_t)kLanes & m;
-    return n;
-}
-
-template <int Q, int QO, int GSUB>
-__device__ __forceinline__ void load_tile(TileRegs<Q, QO, GSUB> &r, const NextTile &n)
-{
-#pragma unroll
-    for (int d = 0; d < GSUB * QO; d++) r.scale[d] = __builtin_nontemporal_load(n.scale + d);
-#pragma unroll
-    for (int u = 0; u < 2 * Q; u++) r.sign[u] = __builtin_nontemporal_load(n.sign + u * n.sign_stride);
-}
-
 // Raw fp16 activations of this lane's chunk in k-block ts (zero beyond k or when !valid).
 // Branch free for the same reason.  x is contiguous.
 __device__ __forceinline__ u32x4 load_activations(const __half *x, int k, int ts, int lane, bool valid)
@@ -483,56 +445,6 @@ __device__ __forceinline__ float reduce_across_lanes(float (&acc)[kBatch], int l
     const unsigned other =
         __builtin_amdgcn_update_dpp(0u, as_u(acc[0]), 0xb1 /* quad_perm:[1,0,3,2] */, 0xf, 0xf, true);
     return acc[0] + as_f(other);
-}
-
-// Lane pair (2j, 2j+1) of a wavefront holds the k-range total of output `out`; the even lane
-// delivers it.  With one k-split it is the result.  Otherwise: one 64-bit atomic add per output,
-// no barrier, no second pass.  The word holds an arrival count in its top 8 bits and the running
-// sum below it, as a biased fixed-point integer (2^-24 units, bias 2^46 per addend so every
-// addend is positive; at most 128 addends below 2^47 keep the sum below 2^54 and out of the
-// flags and the count).  Integer addition is associative, so the total does not depend on the
-// order in which the workgroups arrive: the result is deterministic.  The workgroup whose add
-// returns count == k_splits-1 is the last one for that output: it holds the complete sum, writes
-// y and puts the word back to zero for the next launch.
-// A partial sum that is not finite cannot be expressed in fixed point.  Its workgroup first sets
-// a flag in the same word (bit 54: +infinity seen, bit 55: -infinity seen, both: NaN) and then
-// adds a zero contribution; the finishing workgroup turns the flags into the value IEEE
-// arithmetic gives the sum: +-infinity, or NaN for a NaN or for infinities of both signs.  The
-// flag store and the add are atomics of one thread on one address, so they take effect in
-// program order.
-constexpr unsigned long long kPosInfFlag = 1ull << 54, kNegInfFlag = 1ull << 55;
-__device__ __forceinline__ void finish_output(float total, bool active, int out, int lane, __half *y,
-                                              unsigned long long *accum, const MatvecArgs &a)
-{
-    if (!(active && (lane & 1) == 0 && out < a.n)) return;
-    if (a.k_splits == 1) {
-        y[(size_t)out * a.y_stride] = __float2half_rn(total);
-        return;
-    }
-    unsigned long long *word = accum + out;
-    float scaled = total * 16777216.f;
-    if (!(fabsf(scaled) < 7.0e13f)) {  // beyond 2^46 in fixed point, infinite or NaN
-        const unsigned long long flags =
-            total != total ? (kPosInfFlag | kNegInfFlag) : total > 0.f ? kPosInfFlag : kNegInfFlag;
-        __hip_atomic_fetch_or(word, flags, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        scaled = 0.f;
-    }
-    const unsigned long long addend =
-        (unsigned long long)(__float2ll_rn(scaled) + (1ll << 46)) + (1ull << 56);
-    const unsigned long long old =
-        __hip_atomic_fetch_add(word, addend, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    if ((old >> 56) == (unsigned long long)(a.k_splits - 1)) {
-        const unsigned long long all = old + addend;
-        const long long value = (long long)(all & (kPosInfFlag - 1)) - (long long)a.k_splits * (1ll << 46);
-        float result = __ll2float_rn(value) * (1.f / 16777216.f);
-        const unsigned long long flags = all & (kPosInfFlag | kNegInfFlag);
-        if (flags)
-            result = flags == kPosInfFlag   ? __builtin_inff()
-                     : flags == kNegInfFlag ? -__builtin_inff()
-                                            : __builtin_nanf("");
-        y[(size_t)out * a.y_stride] = __float2half_rn(result);
-        __hip_atomic_store(word, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    }
 }
 
 // Workgroup `block` of one matvec (the body of lut_matvec_kernel and of lut_matvec_multi_kernel).
@@ -754,9 +666,20 @@ __global__ __launch_bounds__(768) void lut_matvec2_kernel(MatvecArgs a)
     const int out = nb * kBatch + (lane >> 1);
     __half *y = reinterpret_cast<__half *>(a.y);
     const float total0 = reduce_across_lanes(acc0, lane);
-    finish_output(total0, active, out, lane, y, a.accum, a);
     const float total1 = reduce_across_lanes(acc1, lane);
-    finish_output(total1, active && a.rows > 1, out, lane, y + a.y_row_stride, a.accum + a.accum_row_stride, a);
+    const bool valid0 = active && (lane & 1) == 0 && out < a.n, valid1 = valid0 && a.rows > 1;
+    __half *y0 = y + (size_t)out * a.y_stride, *y1 = y0 + a.y_row_stride;
+    if (a.k_splits == 1) {
+        if (valid0) *y0 = __float2half_rn(total0);
+        if (valid1) *y1 = __float2half_rn(total1);
+        return;
+    }
+    // both atomics go out before the first answer is looked at
+    unsigned long long *w0 = a.accum + out, *w1 = w0 + a.accum_row_stride;
+    const Arrival r0 = arrive_output(total0, valid0, w0);
+    const Arrival r1 = arrive_output(total1, valid1, w1);
+    complete_output(r0, valid0, w0, y0, a.k_splits);
+    complete_output(r1, valid1, w1, y1, a.k_splits);
 }
 
 // The matvec without its arithmetic: same grid, same tile registers, the same loads in the same

@@ -120,7 +120,7 @@ def test_cfg2_rtn_with_offset_reduced_n(lutgemm, oracle, device):
     W.close()
 
 
-@pytest.mark.parametrize("m", [2, 3, 4, 5, 8])
+@pytest.mark.parametrize("m", [2, 3, 4, 5, 8, 15, 16, 17, 33])
 def test_batched_rows_and_columns(lutgemm, oracle, device, m):
     from lutgemm import synth
     say("case batch", m)
@@ -140,10 +140,11 @@ def test_batched_rows_and_columns(lutgemm, oracle, device, m):
     (2560, 513, 4, 32, False), (96, 33, 4, 96, True), (7168, 224, 3, 128, True), (640, 70, 8, 128, False),
 ])
 def test_row_pairs_equal_single_rows_bit_for_bit(lutgemm, oracle, device, k, n, q, g, offset):
-    """Rows go through the weight two per pass (a last single row if m is odd); each must come
-    out exactly as a one-row launch with the same plan produces it (same tables, same order of
-    accumulation), for every scale layout (g % 128, % 64, % 32), with and without offset, for
-    several plans."""
+    """A two-row pass must give each row exactly as a one-row launch with the same plan produces
+    it (same tables, same order of accumulation), for every scale layout (g % 128, % 64, % 32),
+    with and without offset, for several plans.  Five rows go two per pass as well when the
+    group size is not a multiple of 128 (then equally bit-identical); otherwise the batch kernel
+    takes them in one pass, within the tolerance."""
     from lutgemm import synth
     m = 5
     w, W = make(lutgemm, synth, k, n, q, g, offset=offset, seed=k + q)
@@ -154,9 +155,13 @@ def test_row_pairs_equal_single_rows_bit_for_bit(lutgemm, oracle, device, k, n, 
         W.set_plan(waves, min(ks, (k + 511) // 512))
         y = run_matvec(lutgemm, W, x, device)
         assert_within_tolerance(y, truth, "m=%d plan=%s" % (m, W.plan()))
+        y2 = run_matvec(lutgemm, W, x[:2], device)
         for r in range(m):
             y1 = run_matvec(lutgemm, W, x[r:r + 1], device)
-            assert np.array_equal(y[r].view(np.uint16), y1[0].view(np.uint16)), "row %d plan %s" % (r, W.plan())
+            if r < 2:
+                assert np.array_equal(y2[r].view(np.uint16), y1[0].view(np.uint16)), "row %d of 2, plan %s" % (r, W.plan())
+            if g % 128 != 0:
+                assert np.array_equal(y[r].view(np.uint16), y1[0].view(np.uint16)), "row %d plan %s" % (r, W.plan())
     W.close()
 
 
@@ -180,6 +185,40 @@ def test_many_rows(lutgemm, oracle, device, k, n, q, g, offset):
         assert np.array_equal(y.view(np.uint16), run_matvec(lutgemm, W, x, device).view(np.uint16))
         yc = run_matvec(lutgemm, W, x, device, cols=True)
         assert np.array_equal(y.view(np.uint16), yc.view(np.uint16))
+    W.close()
+
+
+@pytest.mark.parametrize("k,n,q,g,offset", [
+    (1024, 40, 4, 128, True), (2048, 33, 1, 128, False), (1536, 100, 1, 256, True), (640, 70, 2, 128, True),
+    (4096, 96, 4, 4096, False), (896, 513, 3, 128, True), (3072, 1000, 3, 384, False), (12288, 320, 4, 128, True),
+])
+def test_batch_kernel_shapes(lutgemm, oracle, device, k, n, q, g, offset):
+    """Three and more rows with a group size that is a multiple of 128 and up to four planes go
+    through the weight once on the matrix cores: every plane count, with and without offset, k that
+    ends inside a k-block, n that ends inside a batch, one to many k-splits, row counts below, at
+    and above the 16 rows of a pass; deterministic; row- and column-batched forms agree."""
+    from lutgemm import synth
+    w, W = make(lutgemm, synth, k, n, q, g, offset=offset, seed=k + 5 * q)
+    ts = (k + 511) // 512
+    for m, (waves, ks) in zip((3, 7, 16, 20, 4), ((0, 0), (8, 1), (6, 2), (12, ts), (3, 3))):
+        say("case batch kernel", k, n, q, g, offset, m, waves, ks)
+        x = synth.make_x(m, k, seed=n + m)
+        truth = truth_of(oracle, w, x)
+        W.set_plan(waves, min(ks, ts))
+        y = run_matvec(lutgemm, W, x, device)
+        assert_within_tolerance(y, truth, "m=%d plan=%s" % (m, W.plan()))
+        assert np.array_equal(y.view(np.uint16), run_matvec(lutgemm, W, x, device).view(np.uint16))
+        yc = run_matvec(lutgemm, W, x, device, cols=True)
+        assert np.array_equal(y.view(np.uint16), yc.view(np.uint16))
+    # unit activations in a batch: rows of the dequantised weight, bit for bit (sums of a few fp16 numbers are exact)
+    e = np.zeros((5, k), np.float16)
+    rows = [0, 7, k // 2 + 3, k - 1, 129 % k]
+    for i, r in enumerate(rows):
+        e[i, r] = 1
+    ye = run_matvec(lutgemm, W, e, device)
+    dense = oracle.dense_weight_f64(w["bW"], w["alpha"].astype(np.float16),
+                                    w["q_bias"].astype(np.float16) if offset else None)
+    assert np.array_equal(ye.view(np.uint16), dense[rows].astype(np.float16).view(np.uint16))
     W.close()
 
 
@@ -215,9 +254,10 @@ def test_autotune_keeps_results_and_picks_a_valid_plan(lutgemm, oracle, device):
     singles = np.concatenate([run_matvec(lutgemm, W, x[r:r + 1], device) for r in range(5)])
     assert_within_tolerance(singles, truth, "after autotune %s" % plan)
     # two-row passes keep a measured plan of their own; their rows must still equal the one-row launches
-    for m in (2, 3, 5):
-        y = run_matvec(lutgemm, W, x[:m], device)
-        assert np.array_equal(y.view(np.uint16), singles[:m].view(np.uint16)), m
+    y = run_matvec(lutgemm, W, x[:2], device)
+    assert np.array_equal(y.view(np.uint16), singles[:2].view(np.uint16))
+    for m in (3, 5):   # the batch kernel: another order of additions, same tolerance
+        assert_within_tolerance(run_matvec(lutgemm, W, x[:m], device), truth[:m], "m=%d" % m)
     W.close()
 
 
