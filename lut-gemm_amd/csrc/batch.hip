@@ -52,11 +52,11 @@ constexpr int kXRowBytes = kBlockK * 2 + 16;               // one activation row
                                                            // 16 rows read at one column hit 64 different banks
 constexpr int kXBufBytes = kBatchRows * kXRowBytes;        // 16,640
 constexpr int kStageBytes = 1024;                          // per wavefront: [16 outputs][64 chunk positions]
-constexpr int kBatchMaxWaves = 8;                          // the kernel is compiled for at most 512 threads
+constexpr int kScaleAreaBytes = 256 * 5;                   // per wavefront: up to 5 scale words of its 64 lanes, [word][lane]
 
 __host__ __device__ constexpr int batch_lds_bytes(int waves)
 {
-    return kPatternBytes + 2 * kXBufBytes + waves * kStageBytes;
+    return kPatternBytes + 2 * kXBufBytes + waves * (kStageBytes + kScaleAreaBytes);
 }
 
 // 4 x 4 byte transpose among the lanes c, c + 4, c + 8, c + 12 of a 16-lane row: the lane with
@@ -74,22 +74,23 @@ __device__ __forceinline__ uint32_t stride4_transpose(uint32_t v, uint32_t sel1,
 }
 
 // The activation block of k-block ts is 16 rows x 64 chunks = 1024 pieces of 16 bytes; thread tid
-// moves pieces tid and tid + threads (workgroups have exactly 8 wavefronts).
+// moves pieces tid, tid + threads, ... (PIECES = 1024 / threads, rounded up).
 // Loads and LDS writes are separate so that the loads of the next block are in flight while the
 // current one is processed.  Rows beyond the batch and k beyond the weight are zero.
-constexpr int kMaxPieces = 2;
+template <int PIECES>
 struct ActivationPieces {
-    u32x4 v[kMaxPieces];
+    u32x4 v[PIECES];
 };
 
-__device__ __forceinline__ void load_activation_pieces(ActivationPieces &p, const MatvecArgs &a, int ts, int tid,
+template <int PIECES>
+__device__ __forceinline__ void load_activation_pieces(ActivationPieces<PIECES> &p, const MatvecArgs &a, int ts, int tid,
                                                        int threads, bool valid)
 {
     // Branch free (a masked address and masked data instead of a conditional load), so that the
     // compiler's wait counts for the loads around it stay exact.
     const __half *x = reinterpret_cast<const __half *>(a.x);
 #pragma unroll
-    for (int i = 0; i < kMaxPieces; i++) {
+    for (int i = 0; i < PIECES; i++) {
         const int piece = (tid + i * threads) & (kBatchRows * kLanes - 1);
         const int r = piece >> 6, c = piece & 63;
         const int kpos = ts * kBlockK + c * kChunk;
@@ -104,10 +105,11 @@ __device__ __forceinline__ void load_activation_pieces(ActivationPieces &p, cons
     }
 }
 
-__device__ __forceinline__ void store_activation_pieces(const ActivationPieces &p, lds_byte *buf, int tid, int threads)
+template <int PIECES>
+__device__ __forceinline__ void store_activation_pieces(const ActivationPieces<PIECES> &p, lds_byte *buf, int tid, int threads)
 {
 #pragma unroll
-    for (int i = 0; i < kMaxPieces; i++) {
+    for (int i = 0; i < PIECES; i++) {
         const int piece = tid + i * threads;
         const int r = piece >> 6, c = piece & 63;
         if (piece < kBatchRows * kLanes)
@@ -115,8 +117,8 @@ __device__ __forceinline__ void store_activation_pieces(const ActivationPieces &
     }
 }
 
-template <int Q, bool OFF>
-__global__ __launch_bounds__(512) void lut_batch_kernel(MatvecArgs a)
+template <int Q, bool OFF, int W>
+__global__ __launch_bounds__(W * 64) void lut_batch_kernel(MatvecArgs a)
 {
     constexpr int QO = Q + (OFF ? 1 : 0);
     constexpr int NU = 2 * Q;   // sign vectors (units) of a tile: unit U = plane U / 2, output half U % 2
@@ -139,7 +141,8 @@ __global__ __launch_bounds__(512) void lut_batch_kernel(MatvecArgs a)
     const bool active = nb < a.nb;
     const int ts0 = ks * a.blocks_per_split;
     const int ts1 = min(ts0 + a.blocks_per_split, a.ts);
-    lds_byte *stage = lds + kPatternBytes + 2 * kXBufBytes + wave * kStageBytes;
+    lds_byte *stage = lds + kPatternBytes + 2 * kXBufBytes + wave * (kStageBytes + kScaleAreaBytes);
+    lds_byte *scale_area = stage + kStageBytes;
 
     // Sign patterns: entry e, dword v holds the fp16 pair for bits 2v and 2v+1 of e: +1.0 where
     // the bit is set, -1.0 where it is clear.  All 16 lane slots of an entry hold the same 16 bytes.
@@ -152,7 +155,7 @@ __global__ __launch_bounds__(512) void lut_batch_kernel(MatvecArgs a)
         m.w = (((e >> 6) & 1u) ? 0x3c00u : 0xbc00u) | (((e >> 7) & 1u) ? 0x3c000000u : 0xbc000000u);
         *reinterpret_cast<__attribute__((address_space(3))) u32x4 *>(pattern + idx * 16) = m;
     }
-    ActivationPieces pieces;
+    ActivationPieces<(kBatchRows * kLanes + W * kLanes - 1) / (W * kLanes)> pieces;
     load_activation_pieces(pieces, a, ts0, tid, threads, true);
     store_activation_pieces(pieces, xbuf, tid, threads);
 
@@ -173,24 +176,23 @@ __global__ __launch_bounds__(512) void lut_batch_kernel(MatvecArgs a)
     // bytes 0, 2 and 3 of a pattern address: lane slot and the LDS address bits above 64 KiB
     const uint32_t pattern_lane = ((uint32_t)j << 4) + (uint32_t)(size_t)pattern;
 
-    // The sign vectors of a tile as in the one-row kernel.  Scale words: those of ALL four 128-k
-    // groups of the k-block for this lane's two outputs (j and 16 + j); group r is held by lane
-    // 16 r + j of the scale tile.  Both are fetched one k-block ahead.
+    // One tile in registers as in the one-row kernel: the sign vectors and this lane's own scale
+    // words, both fetched one k-block ahead.  The MFMA lanes need the scales of all four 128-k
+    // groups of the k-block for their two outputs (j and 16 + j); group r is held by lane 16 r + j,
+    // so every wavefront passes its scale words through a small LDS area of its own, [word][lane].
     u32x4 sign[NU];
-    uint32_t sc[4][QO];
-    auto scale_address = [&](size_t tile, int r, bool real) {
-        const size_t m = (size_t)0 - (size_t)real;
-        return scales + (((tile * kLanes + 16 * r + j) * (size_t)QO) & m);
-    };
+    uint32_t scale[QO];
     {
         const NextTile n0 = tile_address<Q, QO, 1>(signs, scales, tile0 + ts0, lane, true);
 #pragma unroll
-        for (int r = 0; r < 4; r++)
-#pragma unroll
-            for (int d = 0; d < QO; d++) sc[r][d] = __builtin_nontemporal_load(scale_address(tile0 + ts0, r, true) + d);
+        for (int d = 0; d < QO; d++) scale[d] = __builtin_nontemporal_load(n0.scale + d);
 #pragma unroll
         for (int u = 0; u < NU; u++) sign[u] = __builtin_nontemporal_load(n0.sign + u * n0.sign_stride);
     }
+    __attribute__((address_space(3))) uint32_t *scale_w =
+        reinterpret_cast<__attribute__((address_space(3))) uint32_t *>(scale_area) + lane;
+    const __attribute__((address_space(3))) uint32_t *scale_r =
+        reinterpret_cast<const __attribute__((address_space(3))) uint32_t *>(scale_area) + j;
 
     float4v acc[2];
     acc[0] = float4v{0.f, 0.f, 0.f, 0.f};
@@ -205,19 +207,15 @@ __global__ __launch_bounds__(512) void lut_batch_kernel(MatvecArgs a)
         const NextTile next = tile_address<Q, QO, 1>(signs, scales, tile0 + ts + 1, lane, more);
         load_activation_pieces(pieces, a, ts + 1, tid, threads, more);
 
-        // scale words of this k-block (two fp16 per word), then the refill of their registers
-        uint32_t scw[4][QO];
+        // this k-block's scale words into the wavefront's LDS area, then the refill of their registers
 #pragma unroll
-        for (int r = 0; r < 4; r++)
+        for (int d = 0; d < QO; d++) scale_w[d * kLanes] = scale[d];
 #pragma unroll
-            for (int d = 0; d < QO; d++) scw[r][d] = sc[r][d];
-#pragma unroll
-        for (int r = 0; r < 4; r++)
-#pragma unroll
-            for (int d = 0; d < QO; d++) sc[r][d] = __builtin_nontemporal_load(scale_address(tile0 + ts + 1, r, more) + d);
+        for (int d = 0; d < QO; d++) scale[d] = __builtin_nontemporal_load(next.scale + d);
         // fp16 number hb (= output half * QO + plane-or-offset) of group r as fp32
         auto scale_of = [&](int r, int hb) {
-            const __half2 h2 = *reinterpret_cast<const __half2 *>(&scw[r][hb >> 1]);
+            const uint32_t w = scale_r[(hb >> 1) * kLanes + 16 * r];
+            const __half2 h2 = *reinterpret_cast<const __half2 *>(&w);
             return (hb & 1) ? __high2float(h2) : __low2float(h2);
         };
 
@@ -246,8 +244,8 @@ __global__ __launch_bounds__(512) void lut_batch_kernel(MatvecArgs a)
                     constexpr int t = 4 * r + TT;   // MFMA t: chunks 4 t .. 4 t + 3
                     const half8 xa = *reinterpret_cast<const __attribute__((address_space(3))) half8 *>(xr + t * 64);
                     static_for<CH>([&](auto I) {
-                        constexpr uint32_t sel = 0x03020400u + ((uint32_t)(t & 3) << 8);   // address byte 1 <- sign byte t % 4
                         const uint32_t word = t < 4 ? R[I].x : t < 8 ? R[I].y : t < 12 ? R[I].z : R[I].w;
+                        constexpr uint32_t sel = 0x03020400u + ((uint32_t)(t & 3) << 8);   // address byte 1 <- sign byte t % 4
                         const uint32_t addr = __builtin_amdgcn_perm(word, pattern_lane, sel);
                         const half8 bits = *reinterpret_cast<const __attribute__((address_space(3))) half8 *>(addr);
                         part[I] = __builtin_amdgcn_mfma_f32_16x16x32_f16(xa, bits, TT == 0 ? zero4 : part[I], 0, 0, 0);
@@ -334,8 +332,8 @@ __global__ __launch_bounds__(512) void lut_batch_kernel(MatvecArgs a)
         for (int v = 0; v < 4; v++) complete_output(arrival[h][v], valid[h][v], word[h][v], yout[h][v], a.k_splits);
 }
 
-template <int Q, bool OFF>
-hipError_t launch_batch_q(const MatvecArgs &a, int workgroups, int waves, hipStream_t stream)
+template <int Q, bool OFF, int W>
+hipError_t launch_batch_w(const MatvecArgs &a, int workgroups, hipStream_t stream)
 {
     static std::atomic<unsigned long long> allowed{0};
     int dev = 0;
@@ -343,27 +341,28 @@ hipError_t launch_batch_q(const MatvecArgs &a, int workgroups, int waves, hipStr
     if (e != hipSuccess) return e;
     const unsigned long long bit = 1ull << (dev & 63);
     if (!(allowed.load(std::memory_order_relaxed) & bit)) {
-        e = hipFuncSetAttribute(reinterpret_cast<const void *>(&lut_batch_kernel<Q, OFF>),
-                                hipFuncAttributeMaxDynamicSharedMemorySize, batch_lds_bytes(kBatchMaxWaves));
+        e = hipFuncSetAttribute(reinterpret_cast<const void *>(&lut_batch_kernel<Q, OFF, W>),
+                                hipFuncAttributeMaxDynamicSharedMemorySize, batch_lds_bytes(W));
         if (e != hipSuccess) return e;
         allowed.fetch_or(bit, std::memory_order_relaxed);
     }
-    hipLaunchKernelGGL((lut_batch_kernel<Q, OFF>), dim3(workgroups), dim3(waves * kLanes), batch_lds_bytes(waves), stream,
-                       a);
+    hipLaunchKernelGGL((lut_batch_kernel<Q, OFF, W>), dim3(workgroups), dim3(W * kLanes), batch_lds_bytes(W), stream, a);
     return hipGetLastError();
 }
 
 template <int Q>
 hipError_t launch_batch_off(int has_offset, const MatvecArgs &a, int wg, int waves, hipStream_t s)
 {
-    return has_offset ? launch_batch_q<Q, true>(a, wg, waves, s) : launch_batch_q<Q, false>(a, wg, waves, s);
+    if (waves != batch_waves(Q)) return hipErrorInvalidValue;
+    constexpr int W = batch_waves(Q);
+    return has_offset ? launch_batch_w<Q, true, W>(a, wg, s) : launch_batch_w<Q, false, W>(a, wg, s);
 }
 
 }  // namespace
 
 hipError_t launch_batch(int q, int has_offset, const MatvecArgs &a, int workgroups, int waves, hipStream_t stream)
 {
-    if (a.rows < 1 || a.rows > kBatchRows || waves != kBatchMaxWaves) return hipErrorInvalidValue;
+    if (a.rows < 1 || a.rows > kBatchRows) return hipErrorInvalidValue;
     switch (q) {
         case 1: return launch_batch_off<1>(has_offset, a, workgroups, waves, stream);
         case 2: return launch_batch_off<2>(has_offset, a, workgroups, waves, stream);

@@ -178,31 +178,21 @@ FusedPlan choose_fused_plan(const Shape *const *shapes, int count, int cus)
     return best;
 }
 
-// Launch plan of the batch kernel (3..16 rows per pass on the matrix cores): 8 wavefronts per
-// workgroup; the k-split is chosen so that the rounds of workgroups are full.  Per k-block a
-// workgroup is bound by its LDS reads (16 bytes per lane and sign byte for the matrix operand:
-// 32 q + 16 + 2 q reads of 1 KiB per tile at 128 bytes per clock), not by the stream; start and
-// end of a workgroup (pattern table, first activation block, split-k atomics) cost about 3 us.
+// Launch plan of the batch kernel (3..16 rows per pass on the matrix cores): a fixed number of
+// wavefronts per workgroup (16 up to two planes, 8 beyond: registers per wavefront grow with the
+// planes) and as many k-splits as keep all workgroups resident at once (one per compute unit).
+// The kernel is bound by the matrix and vector instructions per tile, not by the stream, so what
+// matters is an even spread of the tiles over the compute units; measured on the decoder-layer
+// shapes, a single round of workgroups beats several shorter rounds.
 Plan choose_batch_plan(const Shape &s, int cus)
 {
-    const int waves = 8;
+    const int waves = lutgemm_kernels::batch_waves(s.q);
     const int ntiles = div_up(s.nb, waves);
-    const double kClockMHz = 2300.0, kStartEnd = 3.0, kBytesPerCu = 7.0e6 / 256.0;
-    const double t_lds = 1.2 * waves * (34.0 * s.q + 16.0) * 8.0 / kClockMHz;
-    const double t_mem = waves * (double)(sign_tile_bytes(s) + scale_tile_bytes(s)) / kBytesPerCu;
-    const double t_block = t_lds > t_mem ? t_lds : t_mem;
-    Plan best{waves, ntiles, s.ts, 1};
-    double best_cost = 1e300;
-    for (int bps = div_up(s.ts, kMaxSplits); bps <= s.ts; bps++) {
-        const int ks = div_up(s.ts, bps);
-        const long groups = (long)ntiles * ks;
-        const double cost = (double)((groups + cus - 1) / cus) * (bps * t_block + kStartEnd);
-        if (cost < best_cost - 1e-9) {
-            best_cost = cost;
-            best = Plan{waves, ntiles, bps, ks};
-        }
-    }
-    return best;
+    int ks = ntiles < cus ? cus / ntiles : 1;
+    if (ks > s.ts) ks = s.ts;
+    if (ks > kMaxSplits) ks = kMaxSplits;
+    const int bps = div_up(s.ts, ks);
+    return Plan{waves, ntiles, bps, div_up(s.ts, bps)};
 }
 
 // A handle's device memory belongs to the device that was current when it was created.

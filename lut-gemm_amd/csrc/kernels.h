@@ -57,8 +57,10 @@ hipError_t launch_matvec_multi(int q, int has_offset, int gsub, const MultiMatve
                                hipStream_t stream);
 
 // 1..kBatchRows activation rows in one pass (matrix cores); scale layouts with gsub == 1 and up to
-// kBatchMaxPlanes planes only, exactly 8 wavefronts per workgroup.
+// kBatchMaxPlanes planes only; batch_waves(q) wavefronts per workgroup (the more planes, the more
+// registers a wavefront needs and the fewer wavefronts fit a compute unit).
 constexpr int kBatchMaxPlanes = 4;
+constexpr int batch_waves(int q) { return q <= 2 ? 16 : 8; }
 hipError_t launch_batch(int q, int has_offset, const MatvecArgs &a, int workgroups, int waves, hipStream_t stream);
 
 // words[0..count) = 0 (a fill kernel rather than a memset node, so that it can be captured)

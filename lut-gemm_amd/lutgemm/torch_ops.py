@@ -6,9 +6,13 @@
 The operator launches on torch's current stream and allocates nothing but its output, so it can
 be captured into a HIP graph like any other torch op.  Batches larger than `dense_threshold`
 rows go through the dequantised fp16 weight and the library GEMM, the route the reference takes
-for every m > 1 (lutGEMM/src/kernels.cu:73-79); below it the LUT kernel streams the packed
-weight once per two rows.
+for every m > 1 (lutGEMM/src/kernels.cu:73-79); up to it the library streams the packed weight
+(one or two rows through the table-lookup kernels, more through the batch kernel, 16 rows per
+pass).  The default threshold is where two passes of the batch kernel meet a library GEMM over
+the dense weight on MI355X (about 32 rows at k = n = 12288).
 """
+DENSE_THRESHOLD = 32
+
 import weakref
 
 import numpy as np
@@ -65,7 +69,7 @@ class LutLinear(torch.nn.Module):
     container: dict(bW, alpha, q_bias, k, n, q, num_groups) as quantize.to_container returns.
     """
 
-    def __init__(self, container, bias=None, dense_threshold=7, autotune=False):
+    def __init__(self, container, bias=None, dense_threshold=DENSE_THRESHOLD, autotune=False):
         super().__init__()
         c = container
         self.weight = BCQWeight(c["bW"], c["alpha"], c["k"], c["n"], c["q"], c["num_groups"], c.get("q_bias"))
@@ -85,11 +89,16 @@ class LutLinear(torch.nn.Module):
         self = cls.__new__(cls)
         torch.nn.Module.__init__(self)
         self.weight = BCQWeight.load(path)
+        if kw.get("autotune", False):
+            self.weight.autotune(torch.cuda.current_stream().cuda_stream)
         self.handle = register(self.weight)
         self.in_features, self.out_features = self.weight.kSize, self.weight.mSize
-        self.dense_threshold = kw.get("dense_threshold", 7)
+        self.dense_threshold = kw.get("dense_threshold", DENSE_THRESHOLD)
         self._dense = None
-        self.bias = None if bias is None else torch.as_tensor(bias).to(torch.float16).cuda()
+        if bias is not None:
+            self.register_buffer("bias", torch.as_tensor(bias).to(torch.float16).cuda())
+        else:
+            self.bias = None
         return self
 
     @classmethod
@@ -111,8 +120,9 @@ class LutLinear(torch.nn.Module):
 
     def forward(self, x):
         rows = x.numel() // x.shape[-1]
+        x = x.to(torch.float16)
         if rows > self.dense_threshold:
-            y = torch.nn.functional.linear(x.to(torch.float16), self.dense_weight())
+            y = torch.nn.functional.linear(x, self.dense_weight())
         else:
             y = torch.ops.lutgemm.matvec(x, self.handle)
         return y if self.bias is None else y + self.bias

@@ -56,12 +56,13 @@ def test_large_batches_take_the_dense_route(lutgemm, oracle, device):
     assert np.abs(y_dense.cpu().double().numpy() - truth).max() <= 3e-2   # fp16 weight + library GEMM
 
 
-def test_operator_replays_from_a_hip_graph(lutgemm, device):
+@pytest.mark.parametrize("rows", [2, 5])   # the two-row table kernel and the batch kernel
+def test_operator_replays_from_a_hip_graph(lutgemm, device, rows):
     from lutgemm import quantize, torch_ops
     lin, gen = _layer(3, bias=False)
     c, _ = quantize.quantize_linear(lin.weight.detach(), 3, 128, "bcq", rounds=2)
     layer = torch_ops.LutLinear(c)
-    xs = [torch.randn(2, 1024, generator=gen).to(torch.float16).to(device) for _ in range(3)]
+    xs = [torch.randn(rows, 1024, generator=gen).to(torch.float16).to(device) for _ in range(3)]
     eager = [layer(x).clone() for x in xs]
     static_x = xs[0].clone()
     side = torch.cuda.Stream()
