@@ -159,7 +159,9 @@ def _refine(x, B, A, wf=None, use_bst=True):
     levels = A_new @ pats.t()                              # [rows, L]
     lv, order = levels.sort(dim=1)
     mids = ((lv[:, 1:] + lv[:, :-1]) / 2).contiguous()
-    pos = torch.searchsorted(mids, x.contiguous())         # index into the sorted levels
+    # a weight exactly between two levels goes to the upper one, as the `w < mid` test of
+    # examples/bcq.py:177-181 decides
+    pos = torch.searchsorted(mids, x.contiguous(), right=True)   # index into the sorted levels
     which = torch.gather(order, 1, pos)                    # pattern index per weight
     B_new = pats[which]                                    # [rows, g, q]
     if wf is not None:
@@ -217,6 +219,10 @@ def quantize(w, qbits, rounds=15, group_size=-1, transpose=False, exponent=0.0, 
     if qbits > 1:
         for _ in range(rounds):
             B, A = _refine(x, B, A, wf, use_bst)
+    if wf is not None:
+        # pruned weights (factor 0, value set to 0) keep the code 0 in every plane on every route
+        # (the reference's r.sign() of a zero residual, examples/bcq.py:106), not only under use_bst
+        B = B * (wf != 0)[..., None]
     w_hat = torch.einsum("rgq,rq->rg", B, A).reshape(d0, d1)
     if transpose:
         w_hat = w_hat.t().contiguous()

@@ -236,6 +236,32 @@ def test_quantize_options():
     assert (we - w)[big].pow(2).mean() < (wu - w)[big].pow(2).mean()
 
 
+def test_pruned_weights_have_code_zero_on_every_route_and_ties_go_up():
+    """Pruned weights (factor 0, value 0) get 0 in every plane whatever the route (greedy only,
+    greedy sign assignment, nearest level), as r.sign() of a zero residual gives in
+    examples/bcq.py:106; a weight exactly between two levels takes the upper one, as the
+    `w < mid` test of examples/bcq.py:177-181 decides."""
+    from lutgemm import quantize as qz
+    torch.manual_seed(7)
+    w = torch.randn(16, 64)
+    for rounds, use_bst in ((0, True), (3, False), (3, True)):
+        w_hat, binary, alpha, kept = qz.quantize(w, 3, rounds=rounds, group_size=32, pruning=0.3, use_bst=use_bst)
+        kept = kept.reshape(binary.shape[:3])
+        assert (~kept).any() and kept.any()
+        assert bool((binary[~kept] == 0).all()) and bool((binary[kept].abs() == 1).all())
+        assert bool((w_hat.reshape(kept.shape)[~kept] == 0).all())
+    # levels of alpha = (2, 1) are -3, -1, 1, 3 with midpoints -2, 0, 2.  Four weights sit on the
+    # levels and fix the scales; two more sit exactly on midpoints (0 and 2) with a negligible
+    # weight in the least squares: they must take the upper levels 1 and 3.
+    x = torch.tensor([[3.0, 1.0, -1.0, -3.0, 0.0, 2.0]])
+    B = torch.tensor([[[1.0, 1.0], [1.0, -1.0], [-1.0, 1.0], [-1.0, -1.0], [-1.0, 1.0], [1.0, -1.0]]])
+    wf = torch.tensor([[1.0, 1.0, 1.0, 1.0, 1e-12, 1e-12]])
+    B_new, A_new = qz._refine(x, B, torch.tensor([[2.0, 1.0]]), wf)
+    assert torch.allclose(A_new, torch.tensor([[2.0, 1.0]]), atol=1e-4)
+    got = (B_new * A_new[:, None, :]).sum(-1)
+    assert torch.allclose(got, torch.tensor([[3.0, 1.0, -1.0, -3.0, 1.0, 3.0]]), atol=1e-3)
+
+
 def test_packer_known_answer_and_round_trip():
     """examples/utils.py:164-183: entry i*N/8 + j of the flattened tensor is bit i of byte j."""
     b = -torch.ones(2, 8)            # N = 16, two bytes
