@@ -117,7 +117,10 @@ __device__ __forceinline__ void store_activation_pieces(const ActivationPieces<P
     }
 }
 
-template <int Q, bool OFF, int W>
+// W is the largest number of wavefronts a workgroup may have (it sets the register budget), WMIN
+// the smallest: the launch picks the number in between that divides the column batches of the
+// shape best over the compute units.
+template <int Q, bool OFF, int W, int WMIN>
 __global__ __launch_bounds__(W * 64) void lut_batch_kernel(MatvecArgs a)
 {
     constexpr int QO = Q + (OFF ? 1 : 0);
@@ -155,7 +158,7 @@ __global__ __launch_bounds__(W * 64) void lut_batch_kernel(MatvecArgs a)
         m.w = (((e >> 6) & 1u) ? 0x3c00u : 0xbc00u) | (((e >> 7) & 1u) ? 0x3c000000u : 0xbc000000u);
         *reinterpret_cast<__attribute__((address_space(3))) u32x4 *>(pattern + idx * 16) = m;
     }
-    ActivationPieces<(kBatchRows * kLanes + W * kLanes - 1) / (W * kLanes)> pieces;
+    ActivationPieces<(kBatchRows * kLanes + WMIN * kLanes - 1) / (WMIN * kLanes)> pieces;
     load_activation_pieces(pieces, a, ts0, tid, threads, true);
     store_activation_pieces(pieces, xbuf, tid, threads);
 
@@ -332,8 +335,8 @@ __global__ __launch_bounds__(W * 64) void lut_batch_kernel(MatvecArgs a)
         for (int v = 0; v < 4; v++) complete_output(arrival[h][v], valid[h][v], word[h][v], yout[h][v], a.k_splits);
 }
 
-template <int Q, bool OFF, int W>
-hipError_t launch_batch_w(const MatvecArgs &a, int workgroups, hipStream_t stream)
+template <int Q, bool OFF, int W, int WMIN>
+hipError_t launch_batch_w(const MatvecArgs &a, int workgroups, int waves, hipStream_t stream)
 {
     static std::atomic<unsigned long long> allowed{0};
     int dev = 0;
@@ -341,21 +344,22 @@ hipError_t launch_batch_w(const MatvecArgs &a, int workgroups, hipStream_t strea
     if (e != hipSuccess) return e;
     const unsigned long long bit = 1ull << (dev & 63);
     if (!(allowed.load(std::memory_order_relaxed) & bit)) {
-        e = hipFuncSetAttribute(reinterpret_cast<const void *>(&lut_batch_kernel<Q, OFF, W>),
+        e = hipFuncSetAttribute(reinterpret_cast<const void *>(&lut_batch_kernel<Q, OFF, W, WMIN>),
                                 hipFuncAttributeMaxDynamicSharedMemorySize, batch_lds_bytes(W));
         if (e != hipSuccess) return e;
         allowed.fetch_or(bit, std::memory_order_relaxed);
     }
-    hipLaunchKernelGGL((lut_batch_kernel<Q, OFF, W>), dim3(workgroups), dim3(W * kLanes), batch_lds_bytes(W), stream, a);
+    hipLaunchKernelGGL((lut_batch_kernel<Q, OFF, W, WMIN>), dim3(workgroups), dim3(waves * kLanes), batch_lds_bytes(waves),
+                       stream, a);
     return hipGetLastError();
 }
 
 template <int Q>
 hipError_t launch_batch_off(int has_offset, const MatvecArgs &a, int wg, int waves, hipStream_t s)
 {
-    if (waves != batch_waves(Q)) return hipErrorInvalidValue;
-    constexpr int W = batch_waves(Q);
-    return has_offset ? launch_batch_w<Q, true, W>(a, wg, s) : launch_batch_w<Q, false, W>(a, wg, s);
+    constexpr int W = batch_waves(Q), WMIN = batch_waves_min(Q);
+    if (waves < WMIN || waves > W) return hipErrorInvalidValue;
+    return has_offset ? launch_batch_w<Q, true, W, WMIN>(a, wg, waves, s) : launch_batch_w<Q, false, W, WMIN>(a, wg, waves, s);
 }
 
 }  // namespace

@@ -186,13 +186,31 @@ FusedPlan choose_fused_plan(const Shape *const *shapes, int count, int cus)
 // shapes, a single round of workgroups beats several shorter rounds.
 Plan choose_batch_plan(const Shape &s, int cus)
 {
-    const int waves = lutgemm_kernels::batch_waves(s.q);
-    const int ntiles = div_up(s.nb, waves);
-    int ks = ntiles < cus ? cus / ntiles : 1;
-    if (ks > s.ts) ks = s.ts;
-    if (ks > kMaxSplits) ks = kMaxSplits;
-    const int bps = div_up(s.ts, ks);
-    return Plan{waves, ntiles, bps, div_up(s.ts, bps)};
+    // A compute unit holds one workgroup of the batch kernel.  Per k-block the workgroup spends a
+    // fixed time (its wavefronts meet at a barrier, and the work before the table reads does not
+    // overlap them) plus a time per wavefront (the expansion of a tile's signs through LDS), so a
+    // launch takes (rounds of workgroups) x (k-blocks per workgroup x (fixed + wavefronts x time
+    // per tile) + a start-up per workgroup).  The number of wavefronts
+    // is free between batch_waves_min and batch_waves: the one is chosen that spreads the column
+    // batches over the compute units with the least left idle.
+    const int wmax = lutgemm_kernels::batch_waves(s.q), wmin = lutgemm_kernels::batch_waves_min(s.q);
+    const double tile_us = 0.13 * s.q, start_us = 2.0, block_us = 2.4;   // fitted to measured launches
+    Plan best{wmax, div_up(s.nb, wmax), s.ts, 1};
+    double best_cost = 1e30;
+    for (int waves = wmin; waves <= wmax; waves++) {
+        const int ntiles = div_up(s.nb, waves);
+        for (int ks = 1; ks <= s.ts && ks <= kMaxSplits; ks++) {
+            const int bps = div_up(s.ts, ks);
+            if (div_up(s.ts, bps) != ks) continue;
+            const int rounds = div_up(ntiles * ks, cus);
+            const double cost = rounds * (bps * (waves * tile_us + block_us) + start_us) + 0.02 * ks;
+            if (cost < best_cost) {
+                best_cost = cost;
+                best = Plan{waves, ntiles, bps, ks};
+            }
+        }
+    }
+    return best;
 }
 
 // A handle's device memory belongs to the device that was current when it was created.

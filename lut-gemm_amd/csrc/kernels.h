@@ -61,6 +61,7 @@ hipError_t launch_matvec_multi(int q, int has_offset, int gsub, const MultiMatve
 // registers a wavefront needs and the fewer wavefronts fit a compute unit).
 constexpr int kBatchMaxPlanes = 4;
 constexpr int batch_waves(int q) { return q <= 2 ? 16 : 8; }
+constexpr int batch_waves_min(int q) { return q <= 2 ? 8 : q == 3 ? 6 : 8; }
 hipError_t launch_batch(int q, int has_offset, const MatvecArgs &a, int workgroups, int waves, hipStream_t stream);
 
 // words[0..count) = 0 (a fill kernel rather than a memset node, so that it can be captured)
