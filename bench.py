@@ -229,7 +229,7 @@ def point_record(pt, us, us_hot):
             "fused_independent_us_per_matvec": pt.fused_us,
             "fused_independent_pct_hbm_peak": pt.b_w / pt.fused_us / 1e3 / HBM_PEAK_GBS * 100,
             "hot_us_per_matvec": us_hot, "packed_weight_bytes": pt.b_w, "weight_copies_rotated": pt.copies,
-            "plan": pt.plan}
+            "plan_of_one_row_launches" if pt.m > 1 else "plan": pt.plan}
 
 
 def base_line(args, metric, value, us, workload, extra_config=None):
@@ -312,12 +312,7 @@ def run_single(args, lutgemm, synth, torch, dev, stream, name):
     line["parity"] = parity
 
     if args.copy_calibration:
-        src = torch.empty(128 * 1024 * 1024, dtype=torch.float16, device=dev).fill_(1.0)  # 256 MiB
-        dst = torch.empty_like(src)
-        for _ in range(5):
-            torch.mul(src, 1.0, out=dst)  # an ordinary elementwise kernel: reads 256 MiB, writes 256 MiB
-        torch.cuda.synchronize()
-        del src, dst
+        copy_calibration(torch, dev)
 
     dense = None
     if name == "cfg1" and not args.no_dense:
@@ -363,6 +358,17 @@ def run_single(args, lutgemm, synth, torch, dev, stream, name):
         line["cpu_baseline"] = cpu_baseline(synth, cfg, pt.x16, pt.w, truth)
     pt.close()
     return line
+
+
+def copy_calibration(torch, dev):
+    """Five launches of an ordinary elementwise kernel of known size (reads 256 MiB, writes 256 MiB):
+    what FETCH_SIZE and WRITE_SIZE read for it gives the factor between the counters and bytes."""
+    src = torch.empty(128 * 1024 * 1024, dtype=torch.float16, device=dev).fill_(1.0)  # 256 MiB
+    dst = torch.empty_like(src)
+    for _ in range(5):
+        torch.mul(src, 1.0, out=dst)
+    torch.cuda.synchronize()
+    del src, dst
 
 
 def run_cfg3(args, lutgemm, synth, torch, dev, stream):
@@ -462,6 +468,8 @@ def run_cfg4(args, lutgemm, synth, torch, dev, stream):
         gms = event_time_ms(torch, replay, stream)
         graph = {"us_per_layer_step": gms * 1e3 / (reps * copies), "steps_per_graph": copies,
                  "replays_equal_eager": bool(same)}
+    if args.copy_calibration:
+        copy_calibration(torch, dev)
     value = step_bytes / chain_us / 1e3
     line = base_line(args, "µs per decoder layer (QKV+out+FC1+FC2 matvecs) + weight-GB/s, q=2 g=128 m=%d fp16" % m,
                      value, chain_us / 4.0, "cfg4: OPT-175B decoder layer matvecs q=2 g=128 m=%d" % m,

@@ -178,23 +178,25 @@ FusedPlan choose_fused_plan(const Shape *const *shapes, int count, int cus)
     return best;
 }
 
-// Launch plan of the batch kernel (3..16 rows per pass on the matrix cores): a fixed number of
-// wavefronts per workgroup (16 up to two planes, 8 beyond: registers per wavefront grow with the
-// planes) and as many k-splits as keep all workgroups resident at once (one per compute unit).
-// The kernel is bound by the matrix and vector instructions per tile, not by the stream, so what
-// matters is an even spread of the tiles over the compute units; measured on the decoder-layer
-// shapes, a single round of workgroups beats several shorter rounds.
+// Launch plan of the batch kernel (3..16 rows per pass on the matrix cores): wavefronts per
+// workgroup (at most 16 up to two planes, 8 beyond: registers per wavefront grow with the planes)
+// and k-splits.  The kernel is bound by the expansion of the sign bytes through LDS and by the
+// matrix instructions, not by the stream, so what matters is an even spread of the tiles over
+// the compute units; measured on the decoder-layer shapes, a single round of workgroups beats
+// several shorter rounds.
 Plan choose_batch_plan(const Shape &s, int cus)
 {
     // A compute unit holds one workgroup of the batch kernel.  Per k-block the workgroup spends a
     // fixed time (its wavefronts meet at a barrier, and the work before the table reads does not
-    // overlap them) plus a time per wavefront (the expansion of a tile's signs through LDS), so a
-    // launch takes (rounds of workgroups) x (k-blocks per workgroup x (fixed + wavefronts x time
-    // per tile) + a start-up per workgroup).  The number of wavefronts
-    // is free between batch_waves_min and batch_waves: the one is chosen that spreads the column
-    // batches over the compute units with the least left idle.
+    // overlap them) plus a time per wavefront (the expansion of a tile's signs through LDS); per
+    // workgroup a start-up (pattern table, first memory round trip) and an end (split-k atomics).
+    // A second round of workgroups costs more than its sum (the units wait for the slowest of a
+    // round), so plans that keep all workgroups resident at once win where the shape allows one.
+    // The number of wavefronts is free between batch_waves_min and batch_waves: the one is chosen
+    // that spreads the column batches over the compute units with the least left idle.
+    // Constants in microseconds, fitted to measured launches of the decoder-layer shapes.
     const int wmax = lutgemm_kernels::batch_waves(s.q), wmin = lutgemm_kernels::batch_waves_min(s.q);
-    const double tile_us = 0.13 * s.q, start_us = 2.0, block_us = 2.4;   // fitted to measured launches
+    const double tile_us = 0.13 * s.q, block_us = 2.2, start_us = 5.0, round_us = 8.0;
     Plan best{wmax, div_up(s.nb, wmax), s.ts, 1};
     double best_cost = 1e30;
     for (int waves = wmin; waves <= wmax; waves++) {
@@ -203,7 +205,7 @@ Plan choose_batch_plan(const Shape &s, int cus)
             const int bps = div_up(s.ts, ks);
             if (div_up(s.ts, bps) != ks) continue;
             const int rounds = div_up(ntiles * ks, cus);
-            const double cost = rounds * (bps * (waves * tile_us + block_us) + start_us) + 0.02 * ks;
+            const double cost = rounds * (bps * (waves * tile_us + block_us) + start_us) + (rounds - 1) * round_us + 0.02 * ks;
             if (cost < best_cost) {
                 best_cost = cost;
                 best = Plan{waves, ntiles, bps, ks};
