@@ -110,7 +110,7 @@ int lutgemm_matvec(const lutgemm_weight *w, const void *x, void *y, int m, void 
  * capture, tight serving loops, harnesses that forbid hipMalloc.  It has no counterpart in the
  * reference.  Same arguments, same kernels and bit-identical results; the only difference is where
  * the split-k accumulators live: not in the handle's allocation but in a static device array of
- * the library (1 MiB on every device the library runs on, held until the process ends), whose
+ * the library (8 MiB on every device the library runs on, held until the process ends), whose
  * address is looked up once per device.  Limit: n <= 65,536 outputs (LUTGEMM_ERR_UNSUPPORTED
  * beyond).  The call performs no hipMalloc / hipFree and calls no allocating library routine.  All
  * calls on one device share that device's array, whatever the handle or stream: calls that overlap

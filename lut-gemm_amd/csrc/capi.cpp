@@ -460,10 +460,10 @@ int run_matvec(const lutgemm_weight *w, const void *x, void *y, int m, void *str
     int slot = 0;
     if (static_ws) {
         const size_t words = lutgemm_kernels::kStaticSplitKWords;
-        if ((size_t)kTableRows * s.nb * kBatch > words)
+        if ((size_t)kRowsPerPass * s.nb * kBatch > words)
             return fail(LUTGEMM_ERR_UNSUPPORTED,
                         "n=%d is beyond what the static workspace holds (%zu outputs per activation row)", s.n,
-                        words / kTableRows);
+                        words / kRowsPerPass);
         hipError_t es = lutgemm_kernels::static_split_k_words(w->device, &a.accum);
         if (es != hipSuccess) return hip_fail(es, "hipGetSymbolAddress(static split-k words)");
         if (g_static_dirty[w->device]) {  // a launch failed half way through a call: start from zero again
@@ -495,7 +495,7 @@ int run_matvec(const lutgemm_weight *w, const void *x, void *y, int m, void *str
     }
     a.x_row_stride = s.k;
     a.accum_row_stride = (long long)s.nb * kBatch;
-    if (m >= 3 && s.gsub == 1 && s.q <= lutgemm_kernels::kBatchMaxPlanes && !static_ws) {
+    if (m >= 3 && s.gsub == 1 && s.q <= lutgemm_kernels::kBatchMaxPlanes) {
         // up to 16 rows per pass over the weight on the matrix cores
         const Plan plan = choose_batch_plan(s, w->compute_units);
         a.ntiles = plan.ntiles;
@@ -514,7 +514,10 @@ int run_matvec(const lutgemm_weight *w, const void *x, void *y, int m, void *str
                 a.y_row_stride = s.n;
             }
             hipError_t e = lutgemm_kernels::launch_batch(s.q, s.has_offset, a, plan.ntiles * plan.k_splits, plan.waves, st);
-            if (e != hipSuccess) return hip_fail(e, "launch lut_batch_kernel");
+            if (e != hipSuccess) {
+                if (static_ws && r > 0) g_static_dirty[w->device] = true;
+                return hip_fail(e, "launch lut_batch_kernel");
+            }
         }
         return LUTGEMM_OK;
     }

@@ -68,11 +68,12 @@ hipError_t launch_batch(int q, int has_offset, const MatvecArgs &a, int workgrou
 hipError_t launch_fill_zero(unsigned long long *words, size_t count, hipStream_t stream);
 
 // Split-k words of the allocation-free entry point: a static device array of kStaticSplitKWords
-// 64-bit words (1 MiB on every device the library runs on, enough for 65,536 outputs per
-// activation row of a two-row pass), zero at load and zero again after every completed launch.
+// 64-bit words (8 MiB on every device the library runs on, enough for 65,536 outputs per
+// activation row of a pass of kBatchRows rows), zero at load and zero again after every completed
+// launch.
 // Returns its device address on `device`, which must be the current device (0 <= device <
 // kMaxDevices); looked up once per device.
-constexpr size_t kStaticSplitKWords = (size_t)1 << 17;
+constexpr size_t kStaticSplitKWords = (size_t)1 << 20;
 constexpr int kMaxDevices = 64;
 hipError_t static_split_k_words(int device, unsigned long long **words);
 

@@ -1,6 +1,7 @@
 """The allocation-free entry point lutgemm_matvec_static (split-k words in a static device array)
-against lutgemm_matvec on the same inputs, through the C ABI: bit for bit, on two calls in a row,
-the second on a smaller weight, so that words left behind by the first would show."""
+against lutgemm_matvec on the same inputs, through the C ABI: bit for bit, on calls in a row
+(three, two, one and nine activation rows: batch, two-row and one-row kernels), the second on a
+smaller weight than the first, so that words left behind by a call would show in the next."""
 import ctypes
 import sys
 
@@ -28,7 +29,7 @@ def test_static_workspace_entry_point_matches_matvec(lutgemm, oracle, device):
     from gpu_util import assert_within_tolerance
     # first call: k-splits over a wide weight; second call: a smaller weight with other splits
     for (k, n, q, g, off, plan, m) in [(8192, 6000, 3, 128, True, (8, 8), 3), (2048, 1000, 2, 64, False, (3, 4), 2),
-                                        (4096, 4096, 3, 128, False, (0, 0), 1)]:
+                                        (4096, 4096, 3, 128, False, (0, 0), 1), (4096, 2080, 2, 128, False, (0, 0), 9)]:
         print("case static", k, n, q, g, off, plan, m, flush=True)
         sys.stdout.flush()
         w = synth.make_weight(k, n, q, g, offset=off, seed=k + n)
