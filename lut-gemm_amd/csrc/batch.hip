@@ -63,64 +63,46 @@ __host__ __device__ constexpr int batch_lds_bytes(int waves)
 // e = (lane / 4) % 4 ends with byte e of the dwords of those four lanes, in lane order.
 __device__ __forceinline__ uint32_t stride4_transpose(uint32_t v, uint32_t sel1, uint32_t sel2)
 {
-    // partner lane ^ 4: lanes 0-3 and 8-11 of a row fetch from lane + 4, the others from lane - 4
-    const uint32_t p1 = (uint32_t)__builtin_amdgcn_update_dpp(
-        __builtin_amdgcn_update_dpp(0, (int)v, 0x104 /* row_shl:4 */, 0xf, 0x5, false), (int)v, 0x114 /* row_shr:4 */,
-        0xf, 0xa, false);
+    // partner lane ^ 4: lanes 0-3 and 8-11 of a row fetch from lane + 4, the others from lane - 4.
+    // The first move writes every lane (lanes without a source get zero), the second overwrites
+    // banks 1 and 3, so no lane keeps an old value and the destination needs no initialisation.
+    const uint32_t up = (uint32_t)__builtin_amdgcn_mov_dpp((int)v, 0x104 /* row_shl:4 */, 0xf, 0xf, true);
+    const uint32_t p1 = (uint32_t)__builtin_amdgcn_update_dpp((int)up, (int)v, 0x114 /* row_shr:4 */, 0xf, 0xa, false);
     const uint32_t a = __builtin_amdgcn_perm(p1, v, sel1);
-    // partner lane ^ 8: rotate the row by 8
-    const uint32_t p2 = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)a, 0x128 /* row_ror:8 */, 0xf, 0xf, false);
+    // partner lane ^ 8: rotate the row by 8 (every lane has a source)
+    const uint32_t p2 = (uint32_t)__builtin_amdgcn_mov_dpp((int)a, 0x128 /* row_ror:8 */, 0xf, 0xf, true);
     return __builtin_amdgcn_perm(p2, a, sel2);
 }
 
-// The activation block of k-block ts is 16 rows x 64 chunks = 1024 pieces of 16 bytes; thread tid
-// moves pieces tid, tid + threads, ... (PIECES = 1024 / threads, rounded up).
-// Loads and LDS writes are separate so that the loads of the next block are in flight while the
-// current one is processed.  Rows beyond the batch and k beyond the weight are zero.
-template <int PIECES>
-struct ActivationPieces {
-    u32x4 v[PIECES];
-};
-
-template <int PIECES>
-__device__ __forceinline__ void load_activation_pieces(ActivationPieces<PIECES> &p, const MatvecArgs &a, int ts, int tid,
-                                                       int threads, bool valid)
+// The activation block of k-block ts is 16 rows x 64 chunks of 16 bytes.  Wavefront w moves row w
+// (the launch has at least as many wavefronts as the batch has rows), lane = chunk.  The load and
+// the LDS write are separate so that the load of the next block is in flight while the current
+// one is processed.  k beyond the weight reads as zero; rows beyond the batch are never written
+// and keep the zeros the buffers start with.  No branches: a branch in the loop body costs the
+// register allocator dearly, and with straight-line code the wait counts of the loads stay exact.
+__device__ __forceinline__ u32x4 load_activation_row(const MatvecArgs &a, int ts, int wave, int lane, bool valid)
 {
-    // Branch free (a masked address and masked data instead of a conditional load), so that the
-    // compiler's wait counts for the loads around it stay exact.
     const __half *x = reinterpret_cast<const __half *>(a.x);
-#pragma unroll
-    for (int i = 0; i < PIECES; i++) {
-        const int piece = (tid + i * threads) & (kBatchRows * kLanes - 1);
-        const int r = piece >> 6, c = piece & 63;
-        const int kpos = ts * kBlockK + c * kChunk;
-        const uint32_t m = 0u - (uint32_t)(valid && r < a.rows && kpos < a.k);
-        const size_t offset = ((size_t)r * (size_t)a.x_row_stride + (size_t)kpos) & (size_t)(0 - (long long)(m & 1u));
-        u32x4 v = *reinterpret_cast<const u32x4 *>(x + offset);
-        v.x &= m;
-        v.y &= m;
-        v.z &= m;
-        v.w &= m;
-        p.v[i] = v;
-    }
+    const int kpos = ts * kBlockK + lane * kChunk;
+    const uint32_t m = 0u - (uint32_t)(valid && wave < a.rows && kpos < a.k);
+    const size_t offset = ((size_t)wave * (size_t)a.x_row_stride + (size_t)kpos) & (size_t)(0 - (long long)(m & 1u));
+    u32x4 v = *reinterpret_cast<const u32x4 *>(x + offset);
+    v.x &= m;
+    v.y &= m;
+    v.z &= m;
+    v.w &= m;
+    return v;
 }
 
-template <int PIECES>
-__device__ __forceinline__ void store_activation_pieces(const ActivationPieces<PIECES> &p, lds_byte *buf, int tid, int threads)
+__device__ __forceinline__ void store_activation_row(const u32x4 &v, lds_byte *buf, int wave, int lane)
 {
-#pragma unroll
-    for (int i = 0; i < PIECES; i++) {
-        const int piece = tid + i * threads;
-        const int r = piece >> 6, c = piece & 63;
-        if (piece < kBatchRows * kLanes)
-            *reinterpret_cast<__attribute__((address_space(3))) u32x4 *>(buf + r * kXRowBytes + c * 16) = p.v[i];
-    }
+    *reinterpret_cast<__attribute__((address_space(3))) u32x4 *>(buf + wave * kXRowBytes + lane * 16) = v;
 }
 
-// W is the largest number of wavefronts a workgroup may have (it sets the register budget), WMIN
-// the smallest: the launch picks the number in between that divides the column batches of the
-// shape best over the compute units.
-template <int Q, bool OFF, int W, int WMIN>
+// W is the largest number of wavefronts a workgroup may have (it sets the register budget); the
+// launch picks a number up to it (and not below the rows of the batch) that divides the column
+// batches of the shape well over the compute units.
+template <int Q, bool OFF, int W>
 __global__ __launch_bounds__(W * 64) void lut_batch_kernel(MatvecArgs a)
 {
     constexpr int QO = Q + (OFF ? 1 : 0);
@@ -158,9 +140,12 @@ __global__ __launch_bounds__(W * 64) void lut_batch_kernel(MatvecArgs a)
         m.w = (((e >> 6) & 1u) ? 0x3c00u : 0xbc00u) | (((e >> 7) & 1u) ? 0x3c000000u : 0xbc000000u);
         *reinterpret_cast<__attribute__((address_space(3))) u32x4 *>(pattern + idx * 16) = m;
     }
-    ActivationPieces<(kBatchRows * kLanes + WMIN * kLanes - 1) / (WMIN * kLanes)> pieces;
-    load_activation_pieces(pieces, a, ts0, tid, threads, true);
-    store_activation_pieces(pieces, xbuf, tid, threads);
+    // both activation buffers start at zero
+    for (int idx = tid; idx < 2 * kXBufBytes / 16; idx += threads)
+        *reinterpret_cast<__attribute__((address_space(3))) u32x4 *>(xbuf + idx * 16) = u32x4{0u, 0u, 0u, 0u};
+    u32x4 xrow = load_activation_row(a, ts0, wave, lane, true);
+    __syncthreads();   // the zeros are in place before the first rows go on top of them
+    store_activation_row(xrow, xbuf, wave, lane);
 
     const u32x4 *signs = reinterpret_cast<const u32x4 *>(a.signs);
     const uint32_t *scales = reinterpret_cast<const uint32_t *>(a.scales);
@@ -208,7 +193,7 @@ __global__ __launch_bounds__(W * 64) void lut_batch_kernel(MatvecArgs a)
         const int cur = (ts - ts0) & 1;
         const bool more = ts + 1 < ts1;
         const NextTile next = tile_address<Q, QO, 1>(signs, scales, tile0 + ts + 1, lane, more);
-        load_activation_pieces(pieces, a, ts + 1, tid, threads, more);
+        xrow = load_activation_row(a, ts + 1, wave, lane, more);
 
         // this k-block's scale words into the wavefront's LDS area, then the refill of their registers
 #pragma unroll
@@ -297,7 +282,7 @@ __global__ __launch_bounds__(W * 64) void lut_batch_kernel(MatvecArgs a)
                 }
             });
         }
-        store_activation_pieces(pieces, xbuf + (cur ^ 1) * kXBufBytes, tid, threads);
+        store_activation_row(xrow, xbuf + (cur ^ 1) * kXBufBytes, wave, lane);
         __syncthreads();   // the next activation block is in place; this one is no longer read
     }
 
@@ -335,7 +320,7 @@ __global__ __launch_bounds__(W * 64) void lut_batch_kernel(MatvecArgs a)
         for (int v = 0; v < 4; v++) complete_output(arrival[h][v], valid[h][v], word[h][v], yout[h][v], a.k_splits);
 }
 
-template <int Q, bool OFF, int W, int WMIN>
+template <int Q, bool OFF, int W>
 hipError_t launch_batch_w(const MatvecArgs &a, int workgroups, int waves, hipStream_t stream)
 {
     static std::atomic<unsigned long long> allowed{0};
@@ -344,22 +329,22 @@ hipError_t launch_batch_w(const MatvecArgs &a, int workgroups, int waves, hipStr
     if (e != hipSuccess) return e;
     const unsigned long long bit = 1ull << (dev & 63);
     if (!(allowed.load(std::memory_order_relaxed) & bit)) {
-        e = hipFuncSetAttribute(reinterpret_cast<const void *>(&lut_batch_kernel<Q, OFF, W, WMIN>),
+        e = hipFuncSetAttribute(reinterpret_cast<const void *>(&lut_batch_kernel<Q, OFF, W>),
                                 hipFuncAttributeMaxDynamicSharedMemorySize, batch_lds_bytes(W));
         if (e != hipSuccess) return e;
         allowed.fetch_or(bit, std::memory_order_relaxed);
     }
-    hipLaunchKernelGGL((lut_batch_kernel<Q, OFF, W, WMIN>), dim3(workgroups), dim3(waves * kLanes), batch_lds_bytes(waves),
-                       stream, a);
+    hipLaunchKernelGGL((lut_batch_kernel<Q, OFF, W>), dim3(workgroups), dim3(waves * kLanes), batch_lds_bytes(waves), stream,
+                       a);
     return hipGetLastError();
 }
 
 template <int Q>
 hipError_t launch_batch_off(int has_offset, const MatvecArgs &a, int wg, int waves, hipStream_t s)
 {
-    constexpr int W = batch_waves(Q), WMIN = batch_waves_min(Q);
-    if (waves < WMIN || waves > W) return hipErrorInvalidValue;
-    return has_offset ? launch_batch_w<Q, true, W, WMIN>(a, wg, waves, s) : launch_batch_w<Q, false, W, WMIN>(a, wg, waves, s);
+    constexpr int W = kBatchWaves;
+    if (waves < batch_waves_min(a.rows) || waves > W) return hipErrorInvalidValue;
+    return has_offset ? launch_batch_w<Q, true, W>(a, wg, waves, s) : launch_batch_w<Q, false, W>(a, wg, waves, s);
 }
 
 }  // namespace

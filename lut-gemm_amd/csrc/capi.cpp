@@ -179,12 +179,11 @@ FusedPlan choose_fused_plan(const Shape *const *shapes, int count, int cus)
 }
 
 // Launch plan of the batch kernel (3..16 rows per pass on the matrix cores): wavefronts per
-// workgroup (at most 16 up to two planes, 8 beyond: registers per wavefront grow with the planes)
-// and k-splits.  The kernel is bound by the expansion of the sign bytes through LDS and by the
+// workgroup and k-splits.  The kernel is bound by the expansion of the sign bytes through LDS and by the
 // matrix instructions, not by the stream, so what matters is an even spread of the tiles over
 // the compute units; measured on the decoder-layer shapes, a single round of workgroups beats
 // several shorter rounds.
-Plan choose_batch_plan(const Shape &s, int cus)
+Plan choose_batch_plan(const Shape &s, int rows, int cus)
 {
     // A compute unit holds one workgroup of the batch kernel.  Per k-block the workgroup spends a
     // fixed time (its wavefronts meet at a barrier, and the work before the table reads does not
@@ -192,10 +191,11 @@ Plan choose_batch_plan(const Shape &s, int cus)
     // workgroup a start-up (pattern table, first memory round trip) and an end (split-k atomics).
     // A second round of workgroups costs more than its sum (the units wait for the slowest of a
     // round), so plans that keep all workgroups resident at once win where the shape allows one.
-    // The number of wavefronts is free between batch_waves_min and batch_waves: the one is chosen
+    // The number of wavefronts is free between batch_waves_min and kBatchWaves (a wavefront stages
+    // one activation row, so a batch needs at least as many as it has rows): the one is chosen
     // that spreads the column batches over the compute units with the least left idle.
     // Constants in microseconds, fitted to measured launches of the decoder-layer shapes.
-    const int wmax = lutgemm_kernels::batch_waves(s.q), wmin = lutgemm_kernels::batch_waves_min(s.q);
+    const int wmax = lutgemm_kernels::kBatchWaves, wmin = lutgemm_kernels::batch_waves_min(rows);
     const double tile_us = 0.13 * s.q, block_us = 2.2, start_us = 5.0, round_us = 8.0;
     Plan best{wmax, div_up(s.nb, wmax), s.ts, 1};
     double best_cost = 1e30;
@@ -497,7 +497,7 @@ int run_matvec(const lutgemm_weight *w, const void *x, void *y, int m, void *str
     a.accum_row_stride = (long long)s.nb * kBatch;
     if (m >= 3 && s.gsub == 1 && s.q <= lutgemm_kernels::kBatchMaxPlanes) {
         // up to 16 rows per pass over the weight on the matrix cores
-        const Plan plan = choose_batch_plan(s, w->compute_units);
+        const Plan plan = choose_batch_plan(s, m < kRowsPerPass ? m : kRowsPerPass, w->compute_units);
         a.ntiles = plan.ntiles;
         a.k_splits = plan.k_splits;
         a.blocks_per_split = plan.blocks_per_split;
