@@ -16,8 +16,8 @@
 //  * The tiles arrive "k across lanes" (lane = chunk, 16 bytes = 16 outputs).  Per 16-byte sign
 //    vector the wavefront transposes 4 x 4 byte blocks among the lanes c, c+4, c+8, c+12 of a row
 //    (DPP moves and byte permutes), writes four dwords into a 1 KiB staging area in LDS laid out
-//    [output][chunk position (c % 4) * 16 + c / 4] and reads 16 bytes back: lane (kappa, j) then
-//    holds the sign bytes of output j for chunks kappa, kappa + 4, ..., kappa + 60 in MFMA order.
+//    [kappa = c % 4][output][position c / 4] and reads 16 bytes back: lane (kappa, j) then holds
+//    the sign bytes of output j for chunks kappa, kappa + 4, ..., kappa + 60 in MFMA order.
 //  * The A operand is the activation block: lane (kappa, i) holds x[row i][8 k of chunk
 //    4 t + kappa], read from an LDS copy that the workgroup shares (rows beyond the batch are zero).
 //  * After the four MFMAs of a group, the 16 x 16 result (rows x outputs) is multiplied by the
@@ -32,11 +32,16 @@
 #include <hip/hip_runtime.h>
 
 #include <atomic>
+#include <type_traits>
 
 #include "device_util.h"
 #include "kernels.h"
 #include "layout.h"
 #include "tile_device.h"
+
+#ifndef LUTGEMM_BATCH_AHEAD
+#define LUTGEMM_BATCH_AHEAD 1
+#endif
 
 namespace lutgemm_kernels {
 using namespace lutgemm_layout;
@@ -83,7 +88,10 @@ __device__ __forceinline__ uint32_t stride4_transpose(uint32_t v, uint32_t sel1,
 __device__ __forceinline__ u32x4 load_activation_row(const MatvecArgs &a, int ts, int wave, int lane, bool valid)
 {
     const __half *x = reinterpret_cast<const __half *>(a.x);
-    const int kpos = ts * kBlockK + lane * kChunk;
+    // A row is kept in LDS ordered [kappa = chunk % 4][t = chunk / 4]: position L holds chunk
+    // 4 (L % 16) + L / 16, so that the 16-byte reads of the matrix lanes (kappa, j) at step t fall
+    // into bank groups that depend on j and t only (see the read in the kernel).
+    const int kpos = ts * kBlockK + (4 * (lane & 15) + (lane >> 4)) * kChunk;
     const uint32_t m = 0u - (uint32_t)(valid && wave < a.rows && kpos < a.k);
     const size_t offset = ((size_t)wave * (size_t)a.x_row_stride + (size_t)kpos) & (size_t)(0 - (long long)(m & 1u));
     u32x4 v = *reinterpret_cast<const u32x4 *>(x + offset);
@@ -99,6 +107,42 @@ __device__ __forceinline__ void store_activation_row(const u32x4 &v, lds_byte *b
     *reinterpret_cast<__attribute__((address_space(3))) u32x4 *>(buf + wave * kXRowBytes + lane * 16) = v;
 }
 
+// LDS reads whose order and wait counts are fixed by hand.  The compiler waits for every LDS read
+// right before its first use and schedules that use early, which leaves one read in flight per
+// wavefront; the contraction below instead issues the reads of a whole step (one activation
+// operand, one expanded sign operand per unit) one or two steps ahead and waits with the exact
+// count of younger reads (LDS reads of a wavefront return in order).  The asm statements are
+// volatile, so they keep their order among themselves; a result is tied to the wait that covers
+// it by passing through that wait's (or a following empty) asm statement.
+__device__ __forceinline__ half8 lds_read128(uint32_t addr)
+{
+    half8 v;
+    asm volatile("ds_read_b128 %0, %1" : "=v"(v) : "v"(addr));
+    return v;
+}
+template <int OFFSET>
+__device__ __forceinline__ half8 lds_read128_at(uint32_t addr)
+{
+    half8 v;
+    asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(v) : "v"(addr), "n"(OFFSET));
+    return v;
+}
+template <int OFFSET>
+__device__ __forceinline__ uint32_t lds_read32_at(uint32_t addr)
+{
+    uint32_t v;
+    asm volatile("ds_read_b32 %0, %1 offset:%2" : "=v"(v) : "v"(addr), "n"(OFFSET));
+    return v;
+}
+template <int YOUNGER>
+__device__ __forceinline__ void lds_wait(half8 &v)
+{
+    static_assert(YOUNGER >= 0 && YOUNGER <= 15, "lgkmcnt has four bits");
+    asm volatile("s_waitcnt lgkmcnt(%1)" : "+v"(v) : "n"(YOUNGER));
+}
+__device__ __forceinline__ void after_wait(half8 &v) { asm volatile("" : "+v"(v)); }
+__device__ __forceinline__ void after_wait(uint32_t &v) { asm volatile("" : "+v"(v)); }
+
 // W is the largest number of wavefronts a workgroup may have (it sets the register budget); the
 // launch picks a number up to it (and not below the rows of the batch) that divides the column
 // batches of the shape well over the compute units.
@@ -108,6 +152,7 @@ __global__ __launch_bounds__(W * 64) void lut_batch_kernel(MatvecArgs a)
     constexpr int QO = Q + (OFF ? 1 : 0);
     constexpr int NU = 2 * Q;   // sign vectors (units) of a tile: unit U = plane U / 2, output half U % 2
     constexpr int CH = NU <= 6 ? NU : NU % 6 == 0 ? 6 : NU % 5 == 0 ? 5 : NU % 4 == 0 ? 4 : 2;   // units per pass
+    constexpr int P = Q <= 2 ? LUTGEMM_BATCH_AHEAD : 0;   // steps of LDS reads in flight ahead of the matrix instructions (0: the compiler's order)
     // The kernel's only LDS object, so it starts at LDS address 0: pattern addresses are formed
     // from the sign byte and a lane constant alone.
     extern __shared__ __attribute__((aligned(16))) unsigned char lds_generic[];
@@ -155,12 +200,20 @@ __global__ __launch_bounds__(W * 64) void lut_batch_kernel(MatvecArgs a)
     const int kappa = lane >> 4, j = lane & 15;       // MFMA: k group and output column / activation row
     const uint32_t sel1 = (lane & 4) ? 0x03070105u : 0x06020400u;
     const uint32_t sel2 = (lane & 8) ? 0x03020706u : 0x05040100u;
-    // staging: lane (row r, e = (lane / 4) % 4, e0 = lane % 4) writes dword d of a unit to
-    // [output 4 d + e][positions e0 * 16 + 4 r .. + 3]
-    __attribute__((address_space(3))) uint32_t *stage_w = reinterpret_cast<__attribute__((address_space(3))) uint32_t *>(
-        stage + ((lane >> 2) & 3) * 64 + (lane & 3) * 16 + (lane >> 4) * 4);
-    const __attribute__((address_space(3))) u32x4 *stage_r =
-        reinterpret_cast<const __attribute__((address_space(3))) u32x4 *>(stage + j * 64 + kappa * 16);
+    // staging: lane (row r, e = (lane / 4) % 4, e0 = lane % 4) holds in dword d of a transposed unit
+    // the sign bytes of output 4 d + e, chunk class e0 (= kappa of the reader), positions 4 r .. 4 r + 3.
+    // The area is laid out [kappa][output ^ 4 (kappa / 2)][16 positions]: a 16-byte read is served
+    // for 16 lanes at a time that hold all 16 outputs and two neighbouring kappa, so the reads of
+    // a wavefront fall into 16 different bank groups; the 4-byte writes are served for 32 lanes at
+    // a time over 32 banks, where two lanes per bank is the least this transpose allows.
+    // Dword d goes to output slot 4 (d ^ (e0 / 2)) + e: the swap is folded into two lane addresses.
+    const int stage_lane = (lane & 3) * 256 + ((lane >> 2) & 3) * 16 + (lane >> 4) * 4, stage_swap = ((lane >> 1) & 1) * 64;
+    __attribute__((address_space(3))) uint32_t *stage_w0 =
+        reinterpret_cast<__attribute__((address_space(3))) uint32_t *>(stage + stage_lane + stage_swap);
+    __attribute__((address_space(3))) uint32_t *stage_w1 =
+        reinterpret_cast<__attribute__((address_space(3))) uint32_t *>(stage + stage_lane + 64 - stage_swap);
+    const __attribute__((address_space(3))) u32x4 *stage_r = reinterpret_cast<const __attribute__((address_space(3))) u32x4 *>(
+        stage + kappa * 256 + (j ^ (4 * (kappa >> 1))) * 16);
     // bytes 0, 2 and 3 of a pattern address: lane slot and the LDS address bits above 64 KiB
     const uint32_t pattern_lane = ((uint32_t)j << 4) + (uint32_t)(size_t)pattern;
 
@@ -207,7 +260,7 @@ __global__ __launch_bounds__(W * 64) void lut_batch_kernel(MatvecArgs a)
             return (hb & 1) ? __high2float(h2) : __low2float(h2);
         };
 
-        const lds_byte *xr = xbuf + cur * kXBufBytes + j * kXRowBytes + kappa * 16;
+        const lds_byte *xr = xbuf + cur * kXBufBytes + j * kXRowBytes + kappa * 256;
         // The sign vectors are taken CH at a time (all of them up to three planes), so that the
         // registers of a pass stay within the budget for any number of planes.
         static_for<NU / CH>([&](auto C) {
@@ -217,50 +270,114 @@ __global__ __launch_bounds__(W * 64) void lut_batch_kernel(MatvecArgs a)
             static_for<CH>([&](auto I) {
                 constexpr int U = u0 + I;
                 const u32x4 w4 = sign[U];
-                stage_w[0 * 64] = stride4_transpose(w4.x, sel1, sel2);
-                stage_w[1 * 64] = stride4_transpose(w4.y, sel1, sel2);
-                stage_w[2 * 64] = stride4_transpose(w4.z, sel1, sel2);
-                stage_w[3 * 64] = stride4_transpose(w4.w, sel1, sel2);
+                stage_w0[0] = stride4_transpose(w4.x, sel1, sel2);
+                stage_w1[0] = stride4_transpose(w4.y, sel1, sel2);
+                stage_w0[32] = stride4_transpose(w4.z, sel1, sel2);
+                stage_w1[32] = stride4_transpose(w4.w, sel1, sel2);
                 R[I] = *stage_r;
                 sign[U] = __builtin_nontemporal_load(next.sign + U * next.sign_stride);
             });
-            static_for<4>([&](auto G) {   // the four 128-k groups of the k-block
-                constexpr int r = G;
+            if constexpr (P > 0) {
+                // Steps g = 0..15 of the k-block (MFMA t = g: group g / 4): the LDS reads of step
+                // g + P are issued before step g is waited for and contracted.
+                half8 xa[P + 1];
+                half8 bits[P + 1][CH];
+                uint32_t sw[2][QO];   // scale words of a group, read with the last step of the group
                 float4v part[CH];
                 float4v xsum = zero4;
-                static_for<4>([&](auto TT) {
-                    constexpr int t = 4 * r + TT;   // MFMA t: chunks 4 t .. 4 t + 3
-                    const half8 xa = *reinterpret_cast<const __attribute__((address_space(3))) half8 *>(xr + t * 64);
+                const uint32_t xaddr = (uint32_t)(size_t)xr, saddr = (uint32_t)(size_t)scale_r;
+                auto issue = [&](auto Gc) {
+                    constexpr int g = Gc, slot = g % (P + 1);
+                    xa[slot] = lds_read128_at<g * 16>(xaddr);
                     static_for<CH>([&](auto I) {
-                        const uint32_t word = t < 4 ? R[I].x : t < 8 ? R[I].y : t < 12 ? R[I].z : R[I].w;
-                        constexpr uint32_t sel = 0x03020400u + ((uint32_t)(t & 3) << 8);   // address byte 1 <- sign byte t % 4
-                        const uint32_t addr = __builtin_amdgcn_perm(word, pattern_lane, sel);
-                        const half8 bits = *reinterpret_cast<const __attribute__((address_space(3))) half8 *>(addr);
-                        part[I] = __builtin_amdgcn_mfma_f32_16x16x32_f16(xa, bits, TT == 0 ? zero4 : part[I], 0, 0, 0);
+                        const uint32_t word = g < 4 ? R[I].x : g < 8 ? R[I].y : g < 12 ? R[I].z : R[I].w;
+                        constexpr uint32_t sel = 0x03020400u + ((uint32_t)(g & 3) << 8);   // address byte 1 <- sign byte g % 4
+                        bits[slot][I] = lds_read128(__builtin_amdgcn_perm(word, pattern_lane, sel));
                     });
-                    if constexpr (OFF && C == 0 && NU <= 6)
-                        xsum = __builtin_amdgcn_mfma_f32_16x16x32_f16(xa, __builtin_bit_cast(half8, ones), xsum, 0, 0, 0);
-                });
-                static_for<CH>([&](auto I) {
-                    constexpr int U = u0 + I, b = U / 2, h = U % 2;
-                    const float s = scale_of(r, h * QO + b);
-                    acc[h][0] += s * part[I][0];
-                    acc[h][1] += s * part[I][1];
-                    acc[h][2] += s * part[I][2];
-                    acc[h][3] += s * part[I][3];
-                });
-                if constexpr (OFF && C == 0 && NU <= 6) {
+                    if constexpr ((g & 3) == 3)
+                        static_for<QO>([&](auto Wd) { sw[(g >> 2) & 1][Wd] = lds_read32_at<(Wd * kLanes + 16 * (g >> 2)) * 4>(saddr); });
+                };
+                static_for<P>(issue);
+                static_for<16>([&](auto Gc) {
+                    constexpr int g = Gc, r = g >> 2, TT = g & 3, slot = g % (P + 1);
+                    if constexpr (g + P < 16) issue(std::integral_constant<int, (g + P < 16 ? g + P : 0)>{});
+                    // reads younger than those of step g: the steps g + 1 .. g + P that exist
+                    constexpr int last = g + P < 16 ? g + P : 15;
+                    constexpr int younger = (last - g) * (1 + CH) + QO * ((last >> 2) - (g >> 2) + ((last & 3) == 3) - ((g & 3) == 3));
+                    lds_wait<younger>(xa[slot]);
+                    static_for<CH>([&](auto I) {
+                        after_wait(bits[slot][I]);
+                        part[I] = __builtin_amdgcn_mfma_f32_16x16x32_f16(xa[slot], bits[slot][I], TT == 0 ? zero4 : part[I], 0, 0, 0);
+                    });
+                    if constexpr (OFF)
+                        xsum = __builtin_amdgcn_mfma_f32_16x16x32_f16(xa[slot], __builtin_bit_cast(half8, ones),
+                                                                      TT == 0 ? zero4 : xsum, 0, 0, 0);
+                    if constexpr (TT == 3) {
+                        static_for<QO>([&](auto Wd) { after_wait(sw[r & 1][Wd]); });
+                        auto scale_word = [&](int hb) {
+                            const uint32_t w = sw[r & 1][hb >> 1];
+                            const __half2 h2 = *reinterpret_cast<const __half2 *>(&w);
+                            return (hb & 1) ? __high2float(h2) : __low2float(h2);
+                        };
+                        static_for<CH>([&](auto I) {
+                            constexpr int U = u0 + I, b = U / 2, h = U % 2;
+                            const float sc = scale_word(h * QO + b);
+                            acc[h][0] += sc * part[I][0];
+                            acc[h][1] += sc * part[I][1];
+                            acc[h][2] += sc * part[I][2];
+                            acc[h][3] += sc * part[I][3];
+                        });
+                        if constexpr (OFF) {
 #pragma unroll
-                    for (int h = 0; h < 2; h++) {
-                        const float z = scale_of(r, h * QO + Q);
-                        acc[h][0] += z * xsum[0];
-                        acc[h][1] += z * xsum[1];
-                        acc[h][2] += z * xsum[2];
-                        acc[h][3] += z * xsum[3];
+                            for (int h = 0; h < 2; h++) {
+                                const float z = scale_word(h * QO + Q);
+                                acc[h][0] += z * xsum[0];
+                                acc[h][1] += z * xsum[1];
+                                acc[h][2] += z * xsum[2];
+                                acc[h][3] += z * xsum[3];
+                            }
+                        }
                     }
-                }
-                if constexpr (NU > 6) __builtin_amdgcn_sched_barrier(0);   // many planes: keep the groups' registers apart
-            });
+                });
+            } else {
+            static_for<4>([&](auto G) {   // the four 128-k groups of the k-block
+                    constexpr int r = G;
+                    float4v part[CH];
+                    float4v xsum = zero4;
+                    static_for<4>([&](auto TT) {
+                        constexpr int t = 4 * r + TT;   // MFMA t: chunks 4 t .. 4 t + 3
+                        const half8 xa = *reinterpret_cast<const __attribute__((address_space(3))) half8 *>(xr + t * 16);
+                        static_for<CH>([&](auto I) {
+                            const uint32_t word = t < 4 ? R[I].x : t < 8 ? R[I].y : t < 12 ? R[I].z : R[I].w;
+                            constexpr uint32_t sel = 0x03020400u + ((uint32_t)(t & 3) << 8);   // address byte 1 <- sign byte t % 4
+                            const uint32_t addr = __builtin_amdgcn_perm(word, pattern_lane, sel);
+                            const half8 bits = *reinterpret_cast<const __attribute__((address_space(3))) half8 *>(addr);
+                            part[I] = __builtin_amdgcn_mfma_f32_16x16x32_f16(xa, bits, TT == 0 ? zero4 : part[I], 0, 0, 0);
+                        });
+                        if constexpr (OFF && C == 0 && NU <= 6)
+                            xsum = __builtin_amdgcn_mfma_f32_16x16x32_f16(xa, __builtin_bit_cast(half8, ones), xsum, 0, 0, 0);
+                    });
+                    static_for<CH>([&](auto I) {
+                        constexpr int U = u0 + I, b = U / 2, h = U % 2;
+                        const float s = scale_of(r, h * QO + b);
+                        acc[h][0] += s * part[I][0];
+                        acc[h][1] += s * part[I][1];
+                        acc[h][2] += s * part[I][2];
+                        acc[h][3] += s * part[I][3];
+                    });
+                    if constexpr (OFF && C == 0 && NU <= 6) {
+#pragma unroll
+                        for (int h = 0; h < 2; h++) {
+                            const float z = scale_of(r, h * QO + Q);
+                            acc[h][0] += z * xsum[0];
+                            acc[h][1] += z * xsum[1];
+                            acc[h][2] += z * xsum[2];
+                            acc[h][3] += z * xsum[3];
+                        }
+                    }
+                    if constexpr (NU > 6) __builtin_amdgcn_sched_barrier(0);   // many planes: keep the groups' registers apart
+                });
+            }
             __builtin_amdgcn_sched_barrier(0);   // one pass after the other: keeps the registers of a pass apart
         });
         if constexpr (OFF && NU > 6) {   // many planes: the offset term in a pass of its own
@@ -269,7 +386,7 @@ __global__ __launch_bounds__(W * 64) void lut_batch_kernel(MatvecArgs a)
                 float4v xsum = zero4;
                 static_for<4>([&](auto TT) {
                     constexpr int t = 4 * r + TT;
-                    const half8 xa = *reinterpret_cast<const __attribute__((address_space(3))) half8 *>(xr + t * 64);
+                    const half8 xa = *reinterpret_cast<const __attribute__((address_space(3))) half8 *>(xr + t * 16);
                     xsum = __builtin_amdgcn_mfma_f32_16x16x32_f16(xa, __builtin_bit_cast(half8, ones), xsum, 0, 0, 0);
                 });
 #pragma unroll
