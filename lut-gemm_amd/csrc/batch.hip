@@ -14,10 +14,11 @@
 //    MFMA t of a k-block, chunk 4 t + kappa: the four k groups of an MFMA are four neighbouring
 //    chunks, so an MFMA never mixes two scale groups and four MFMAs cover one 128-k group.
 //  * The tiles arrive "k across lanes" (lane = chunk, 16 bytes = 16 outputs).  Per 16-byte sign
-//    vector the wavefront transposes 4 x 4 byte blocks among the lanes c, c+4, c+8, c+12 of a row
-//    (DPP moves and byte permutes), writes four dwords into a 1 KiB staging area in LDS laid out
-//    [kappa = c % 4][output][position c / 4] and reads 16 bytes back: lane (kappa, j) then holds
-//    the sign bytes of output j for chunks kappa, kappa + 4, ..., kappa + 60 in MFMA order.
+//    vector the wavefront writes its 64 x 16 bytes into a 1 KiB staging area of its own in LDS and
+//    reads them back with two transposing reads (ds_read_b64_tr_b8, a gfx950 instruction: 16 lanes
+//    exchange the bytes of their 8-byte rows inside the LDS unit): lane (kappa, j) then holds the
+//    sign bytes of output j for chunks kappa, kappa + 4, ..., kappa + 60 in MFMA order.  No vector
+//    instruction takes part in the transposition.
 //  * The A operand is the activation block: lane (kappa, i) holds x[row i][8 k of chunk
 //    4 t + kappa], read from an LDS copy that the workgroup shares (rows beyond the batch are zero).
 //  * After the four MFMAs of a group, the 16 x 16 result (rows x outputs) is multiplied by the
@@ -62,21 +63,6 @@ constexpr int kScaleAreaBytes = 256 * 5;                   // per wavefront: up 
 __host__ __device__ constexpr int batch_lds_bytes(int waves)
 {
     return kPatternBytes + 2 * kXBufBytes + waves * (kStageBytes + kScaleAreaBytes);
-}
-
-// 4 x 4 byte transpose among the lanes c, c + 4, c + 8, c + 12 of a 16-lane row: the lane with
-// e = (lane / 4) % 4 ends with byte e of the dwords of those four lanes, in lane order.
-__device__ __forceinline__ uint32_t stride4_transpose(uint32_t v, uint32_t sel1, uint32_t sel2)
-{
-    // partner lane ^ 4: lanes 0-3 and 8-11 of a row fetch from lane + 4, the others from lane - 4.
-    // The first move writes every lane (lanes without a source get zero), the second overwrites
-    // banks 1 and 3, so no lane keeps an old value and the destination needs no initialisation.
-    const uint32_t up = (uint32_t)__builtin_amdgcn_mov_dpp((int)v, 0x104 /* row_shl:4 */, 0xf, 0xf, true);
-    const uint32_t p1 = (uint32_t)__builtin_amdgcn_update_dpp((int)up, (int)v, 0x114 /* row_shr:4 */, 0xf, 0xa, false);
-    const uint32_t a = __builtin_amdgcn_perm(p1, v, sel1);
-    // partner lane ^ 8: rotate the row by 8 (every lane has a source)
-    const uint32_t p2 = (uint32_t)__builtin_amdgcn_mov_dpp((int)a, 0x128 /* row_ror:8 */, 0xf, 0xf, true);
-    return __builtin_amdgcn_perm(p2, a, sel2);
 }
 
 // The activation block of k-block ts is 16 rows x 64 chunks of 16 bytes.  Wavefront w moves row w
@@ -174,6 +160,24 @@ __global__ __launch_bounds__(W * 64) void lut_batch_kernel(MatvecArgs a)
     lds_byte *stage = lds + kPatternBytes + 2 * kXBufBytes + wave * (kStageBytes + kScaleAreaBytes);
     lds_byte *scale_area = stage + kStageBytes;
 
+    const u32x4 *signs = reinterpret_cast<const u32x4 *>(a.signs);
+    const uint32_t *scales = reinterpret_cast<const uint32_t *>(a.scales);
+    const size_t tile0 = (size_t)(active ? nb : 0) * a.ts;
+
+    // One tile in registers as in the one-row kernel: the sign vectors and this lane's own scale
+    // words, both fetched one k-block ahead.  The MFMA lanes need the scales of all four 128-k
+    // groups of the k-block for their two outputs (j and 16 + j); group r is held by lane 16 r + j,
+    // so every wavefront passes its scale words through a small LDS area of its own, [word][lane].
+    u32x4 sign[NU];
+    uint32_t scale[QO];
+    {
+        const NextTile n0 = tile_address<Q, QO, 1>(signs, scales, tile0 + ts0, lane, true);
+#pragma unroll
+        for (int d = 0; d < QO; d++) scale[d] = __builtin_nontemporal_load(n0.scale + d);
+#pragma unroll
+        for (int u = 0; u < NU; u++) sign[u] = __builtin_nontemporal_load(n0.sign + u * n0.sign_stride);
+    }
+    __builtin_amdgcn_sched_barrier(0);
     // Sign patterns: entry e, dword v holds the fp16 pair for bits 2v and 2v+1 of e: +1.0 where
     // the bit is set, -1.0 where it is clear.  All 16 lane slots of an entry hold the same 16 bytes.
     for (int idx = tid; idx < 256 * 16; idx += threads) {
@@ -192,44 +196,33 @@ __global__ __launch_bounds__(W * 64) void lut_batch_kernel(MatvecArgs a)
     __syncthreads();   // the zeros are in place before the first rows go on top of them
     store_activation_row(xrow, xbuf, wave, lane);
 
-    const u32x4 *signs = reinterpret_cast<const u32x4 *>(a.signs);
-    const uint32_t *scales = reinterpret_cast<const uint32_t *>(a.scales);
-    const size_t tile0 = (size_t)(active ? nb : 0) * a.ts;
 
     // lane roles
     const int kappa = lane >> 4, j = lane & 15;       // MFMA: k group and output column / activation row
-    const uint32_t sel1 = (lane & 4) ? 0x03070105u : 0x06020400u;
-    const uint32_t sel2 = (lane & 8) ? 0x03020706u : 0x05040100u;
-    // staging: lane (row r, e = (lane / 4) % 4, e0 = lane % 4) holds in dword d of a transposed unit
-    // the sign bytes of output 4 d + e, chunk class e0 (= kappa of the reader), positions 4 r .. 4 r + 3.
-    // The area is laid out [kappa][output ^ 4 (kappa / 2)][16 positions]: a 16-byte read is served
-    // for 16 lanes at a time that hold all 16 outputs and two neighbouring kappa, so the reads of
-    // a wavefront fall into 16 different bank groups; the 4-byte writes are served for 32 lanes at
-    // a time over 32 banks, where two lanes per bank is the least this transpose allows.
-    // Dword d goes to output slot 4 (d ^ (e0 / 2)) + e: the swap is folded into two lane addresses.
-    const int stage_lane = (lane & 3) * 256 + ((lane >> 2) & 3) * 16 + (lane >> 4) * 4, stage_swap = ((lane >> 1) & 1) * 64;
-    __attribute__((address_space(3))) uint32_t *stage_w0 =
-        reinterpret_cast<__attribute__((address_space(3))) uint32_t *>(stage + stage_lane + stage_swap);
-    __attribute__((address_space(3))) uint32_t *stage_w1 =
-        reinterpret_cast<__attribute__((address_space(3))) uint32_t *>(stage + stage_lane + 64 - stage_swap);
-    const __attribute__((address_space(3))) u32x4 *stage_r = reinterpret_cast<const __attribute__((address_space(3))) u32x4 *>(
-        stage + kappa * 256 + (j ^ (4 * (kappa >> 1))) * 16);
+    // Staging.  ds_read_b64_tr_b8 works on rows of 16 lanes: every lane passes the address of an
+    // 8-byte row, and lane 8 h + b of the 16 receives byte b of the rows addressed by lanes h, h + 2,
+    // ..., h + 14, in that order (measured on gfx950 with tagged bytes).  Lane (kappa, s) addresses
+    // outputs 8 (s % 2) .. 8 (s % 2) + 7 of chunk kappa + 4 (s / 2); lane (kappa, j) then receives
+    // the sign bytes of output j for chunks kappa + 4 t, t = 0..7, and the same read 512 bytes
+    // further on delivers t = 8..15: together the 16 bytes the contraction consumes.
+    // Lane c (chunk c: kap = c % 4, t = c / 4) writes its 16 bytes to the 16-byte slot
+    //     16 (2 (t / 8) + kap / 2) + ((2 (t % 8) + kap % 2) xor 8 (kap / 2)),
+    // chosen so that both directions are free of bank conflicts: the 16 lanes the LDS serves together
+    // on a 16-byte write fall into 16 different slots modulo 16, and the 32 lanes it serves together
+    // on an 8-byte read cover 256 consecutive bytes.
+    const int w_kap = lane & 3, w_t = lane >> 2;
+    const int w_slot = 16 * (2 * (w_t >> 3) + (w_kap >> 1)) + (((2 * (w_t & 7)) + (w_kap & 1)) ^ (8 * (w_kap >> 1)));
+    __attribute__((address_space(3))) u32x4 *stage_w =
+        reinterpret_cast<__attribute__((address_space(3))) u32x4 *>(stage + 16 * w_slot);
+    const int r_slot = 16 * (kappa >> 1) + (((2 * (j >> 1)) + (kappa & 1)) ^ (8 * (kappa >> 1)));
+    typedef int v2i __attribute__((ext_vector_type(2)));
+    __attribute__((address_space(3))) v2i *stage_r0 =
+        reinterpret_cast<__attribute__((address_space(3))) v2i *>(stage + 16 * r_slot + 8 * (j & 1));
+    __attribute__((address_space(3))) v2i *stage_r1 =
+        reinterpret_cast<__attribute__((address_space(3))) v2i *>(stage + 16 * r_slot + 8 * (j & 1) + 512);
     // bytes 0, 2 and 3 of a pattern address: lane slot and the LDS address bits above 64 KiB
     const uint32_t pattern_lane = ((uint32_t)j << 4) + (uint32_t)(size_t)pattern;
 
-    // One tile in registers as in the one-row kernel: the sign vectors and this lane's own scale
-    // words, both fetched one k-block ahead.  The MFMA lanes need the scales of all four 128-k
-    // groups of the k-block for their two outputs (j and 16 + j); group r is held by lane 16 r + j,
-    // so every wavefront passes its scale words through a small LDS area of its own, [word][lane].
-    u32x4 sign[NU];
-    uint32_t scale[QO];
-    {
-        const NextTile n0 = tile_address<Q, QO, 1>(signs, scales, tile0 + ts0, lane, true);
-#pragma unroll
-        for (int d = 0; d < QO; d++) scale[d] = __builtin_nontemporal_load(n0.scale + d);
-#pragma unroll
-        for (int u = 0; u < NU; u++) sign[u] = __builtin_nontemporal_load(n0.sign + u * n0.sign_stride);
-    }
     __attribute__((address_space(3))) uint32_t *scale_w =
         reinterpret_cast<__attribute__((address_space(3))) uint32_t *>(scale_area) + lane;
     const __attribute__((address_space(3))) uint32_t *scale_r =
@@ -265,16 +258,16 @@ __global__ __launch_bounds__(W * 64) void lut_batch_kernel(MatvecArgs a)
         // registers of a pass stay within the budget for any number of planes.
         static_for<NU / CH>([&](auto C) {
             constexpr int u0 = C * CH;
-            // transpose; the registers of a sign vector are refilled right away
+            // transpose through the staging area (LDS operations of a wavefront execute in order, so
+            // the reads see the write before them and the next write comes after them); the registers
+            // of a sign vector are refilled right away
             u32x4 R[CH];
             static_for<CH>([&](auto I) {
                 constexpr int U = u0 + I;
-                const u32x4 w4 = sign[U];
-                stage_w0[0] = stride4_transpose(w4.x, sel1, sel2);
-                stage_w1[0] = stride4_transpose(w4.y, sel1, sel2);
-                stage_w0[32] = stride4_transpose(w4.z, sel1, sel2);
-                stage_w1[32] = stride4_transpose(w4.w, sel1, sel2);
-                R[I] = *stage_r;
+                *stage_w = sign[U];
+                const v2i lo = __builtin_amdgcn_ds_read_tr8_b64_v2i32(stage_r0);
+                const v2i hi = __builtin_amdgcn_ds_read_tr8_b64_v2i32(stage_r1);
+                R[I] = u32x4{(uint32_t)lo.x, (uint32_t)lo.y, (uint32_t)hi.x, (uint32_t)hi.y};
                 sign[U] = __builtin_nontemporal_load(next.sign + U * next.sign_stride);
             });
             if constexpr (P > 0) {
