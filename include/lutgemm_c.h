@@ -197,7 +197,8 @@ int lutgemm_weight_set_plan(lutgemm_weight *w, int waves_per_group, int k_splits
 /* Measure the most promising launch plans on the device (a few launches each, on `stream`, with
  * scratch activations of its own) and keep the fastest, separately for launches with one
  * activation row and for two-row passes (which keep the k-split of the one-row plan, so that
- * rows stay bit-identical to their own one-row launches).  Optional: the automatic plan is chosen
+ * rows stay bit-identical to their own one-row launches), and, where the batch kernel takes the
+ * shape, for its passes of up to 8 and of 9 to 16 rows.  Optional: the automatic plan is chosen
  * from a model, this replaces it by a measurement.  The measurement streams the weight from
  * HBM as a decoder does: it rotates over temporary device copies of the packed weight (about
  * 1 GiB in total, at most 64 copies) so that no launch finds its weight in the memory-side

@@ -77,6 +77,10 @@ struct lutgemm_weight {
     int xrows_cols;               //   xrows_cols rows of k halves; grown on demand beyond that
     Plan plan;                    // launches with one activation row
     Plan plan2;                   // passes over two activation rows (m >= 2): same k-split as plan
+    // Batch kernel (3 or more rows): measured plans for passes of up to 8 rows [0] and of 9..16 rows
+    // [1], valid when batch_measured[i]; otherwise the model's choice is taken.
+    Plan plan_batch[2];
+    bool batch_measured[2];
 };
 
 namespace {
@@ -179,40 +183,56 @@ FusedPlan choose_fused_plan(const Shape *const *shapes, int count, int cus)
 }
 
 // Launch plan of the batch kernel (3..16 rows per pass on the matrix cores): wavefronts per
-// workgroup and k-splits.  The kernel is bound by the expansion of the sign bytes through LDS and by the
-// matrix instructions, not by the stream, so what matters is an even spread of the tiles over
-// the compute units; measured on the decoder-layer shapes, a single round of workgroups beats
-// several shorter rounds.
+// workgroup and k-splits.  The kernel is bound on the compute units (matrix and vector instruction
+// issue, expansion of the sign bytes through LDS), not by the stream, so what matters is an even
+// spread of the tiles over the compute units.
+// Cost model in microseconds (-1 when `ks` names the same plan as a smaller number of k-splits).
+// A compute unit holds one workgroup.  Per k-block the workgroup spends a fixed time (its
+// wavefronts meet at a barrier) plus a time per wavefront (one tile each); per workgroup a start
+// (launch, pattern table, first memory round trip) and an end (eight split-k atomics per lane: 3 to
+// 5 microseconds of a launch, whatever its shape).  A second round of workgroups costs more than its
+// sum (the units wait for the slowest of a round), so plans that keep all workgroups resident at
+// once win where the shape allows one.  Constants fitted to measured launches of the decoder-layer
+// shapes (k = 12288 or 49152, n = 12288 .. 49152, two planes, eight rows).
+double batch_plan_cost(const Shape &s, int cus, int waves, int ks, Plan *out)
+{
+    const double tile_us = 0.0635 * s.q, block_us = 1.82, start_us = 11.4, round_us = 8.0;
+    const int ntiles = div_up(s.nb, waves);
+    const int bps = div_up(s.ts, ks);
+    if (div_up(s.ts, bps) != ks) return -1.0;
+    const long wgs = (long)ntiles * ks;
+    const int rounds = (int)((wgs + cus - 1) / cus);
+    *out = Plan{waves, ntiles, bps, ks};
+    return rounds * (bps * (waves * tile_us + block_us) + start_us) + (rounds - 1) * round_us + 0.02 * ks;
+}
+
 Plan choose_batch_plan(const Shape &s, int rows, int cus)
 {
-    // A compute unit holds one workgroup of the batch kernel.  Per k-block the workgroup spends a
-    // fixed time (its wavefronts meet at a barrier, and the work before the table reads does not
-    // overlap them) plus a time per wavefront (the expansion of a tile's signs through LDS); per
-    // workgroup a start-up (pattern table, first memory round trip) and an end (split-k atomics).
-    // A second round of workgroups costs more than its sum (the units wait for the slowest of a
-    // round), so plans that keep all workgroups resident at once win where the shape allows one.
-    // The number of wavefronts is free between batch_waves_min and kBatchWaves (a wavefront stages
-    // one activation row, so a batch needs at least as many as it has rows): the one is chosen
-    // that spreads the column batches over the compute units with the least left idle.
-    // Constants in microseconds, fitted to measured launches of the decoder-layer shapes.
     const int wmax = lutgemm_kernels::kBatchWaves, wmin = lutgemm_kernels::batch_waves_min(rows);
-    const double tile_us = 0.13 * s.q, block_us = 2.2, start_us = 5.0, round_us = 8.0;
     Plan best{wmax, div_up(s.nb, wmax), s.ts, 1};
     double best_cost = 1e30;
-    for (int waves = wmin; waves <= wmax; waves++) {
-        const int ntiles = div_up(s.nb, waves);
+    long best_wgs = 0;
+    for (int waves = wmin; waves <= wmax; waves++)
         for (int ks = 1; ks <= s.ts && ks <= kMaxSplits; ks++) {
-            const int bps = div_up(s.ts, ks);
-            if (div_up(s.ts, bps) != ks) continue;
-            const int rounds = div_up(ntiles * ks, cus);
-            const double cost = rounds * (bps * (waves * tile_us + block_us) + start_us) + (rounds - 1) * round_us + 0.02 * ks;
-            if (cost < best_cost) {
-                best_cost = cost;
-                best = Plan{waves, ntiles, bps, ks};
+            Plan p;
+            const double cost = batch_plan_cost(s, cus, waves, ks, &p);
+            if (cost < 0.0) continue;
+            const long wgs = (long)p.ntiles * p.k_splits;
+            // plans the model puts within 4 % of each other: the one that keeps more compute
+            // units busy in a single round has measured better
+            const bool tie = wgs <= cus && best_wgs <= cus && cost < best_cost * 1.04 && cost > best_cost * 0.96;
+            if (tie ? wgs > best_wgs : cost < best_cost) {
+                if (cost < best_cost) best_cost = cost;
+                best = p;
+                best_wgs = wgs;
             }
         }
-    }
     return best;
+}
+
+bool batch_kernel_takes(const Shape &s)
+{
+    return s.gsub == 1 && s.q <= lutgemm_kernels::kBatchMaxPlanes;
 }
 
 // A handle's device memory belongs to the device that was current when it was created.
@@ -307,6 +327,7 @@ int create_from_tiles(const Shape &s, const void *signs, const void *scales, hip
     }
     if (st == LUTGEMM_OK) {
         w->plan = w->plan2 = choose_plan(s, w->compute_units);
+        w->batch_measured[0] = w->batch_measured[1] = false;
         st = alloc_workspace(w);
     }
     if (st != LUTGEMM_OK) {
@@ -495,9 +516,11 @@ int run_matvec(const lutgemm_weight *w, const void *x, void *y, int m, void *str
     }
     a.x_row_stride = s.k;
     a.accum_row_stride = (long long)s.nb * kBatch;
-    if (m >= 3 && s.gsub == 1 && s.q <= lutgemm_kernels::kBatchMaxPlanes) {
+    if (m >= 3 && batch_kernel_takes(s)) {
         // up to 16 rows per pass over the weight on the matrix cores
-        const Plan plan = choose_batch_plan(s, m < kRowsPerPass ? m : kRowsPerPass, w->compute_units);
+        const int pass_rows = m < kRowsPerPass ? m : kRowsPerPass;
+        const Plan plan = w->batch_measured[pass_rows > 8] ? w->plan_batch[pass_rows > 8]
+                                                            : choose_batch_plan(s, pass_rows, w->compute_units);
         a.ntiles = plan.ntiles;
         a.k_splits = plan.k_splits;
         a.blocks_per_split = plan.blocks_per_split;
@@ -592,6 +615,10 @@ int lutgemm_weight_clone(const lutgemm_weight *w, lutgemm_weight **out)
     if (st == LUTGEMM_OK) {
         (*out)->plan = w->plan;
         (*out)->plan2 = w->plan2;
+        for (int i = 0; i < 2; i++) {
+            (*out)->plan_batch[i] = w->plan_batch[i];
+            (*out)->batch_measured[i] = w->batch_measured[i];
+        }
     }
     return st;
 }
@@ -960,17 +987,27 @@ int lutgemm_weight_autotune(lutgemm_weight *w, void *stream)
     void *x = nullptr, *y = nullptr;
     hipEvent_t e0 = nullptr, e1 = nullptr;
     int status = LUTGEMM_OK;
-    hipError_t e = hipMalloc(&x, (size_t)2 * s.k * 2);
-    if (e == hipSuccess) e = hipMalloc(&y, (size_t)2 * s.n * 2);
-    if (e == hipSuccess) e = hipMemsetAsync(x, 0, (size_t)2 * s.k * 2, st);
+    const size_t max_rows = batch_kernel_takes(s) ? (size_t)kRowsPerPass : (size_t)kTableRows;
+    hipError_t e = hipMalloc(&x, max_rows * s.k * 2);
+    if (e == hipSuccess) e = hipMalloc(&y, max_rows * s.n * 2);
+    if (e == hipSuccess) e = hipMemsetAsync(x, 0, max_rows * s.k * 2, st);
     if (e == hipSuccess) e = hipEventCreate(&e0);
     if (e == hipSuccess) e = hipEventCreate(&e1);
     if (e != hipSuccess) status = hip_fail(e, "autotune setup");
     const Plan before = w->plan, before2 = w->plan2;
+    const Plan before_batch[2] = {w->plan_batch[0], w->plan_batch[1]};
+    const bool before_measured[2] = {w->batch_measured[0], w->batch_measured[1]};
     size_t turn = 0;
     // time `reps` launches over `rows` activation rows with plan p, rotating over the copies
     auto measure = [&](const Plan &p, int rows, int reps, float *ms_out) -> int {
-        for (lutgemm_weight *c : copies) (rows == 2 ? c->plan2 : c->plan) = p;
+        for (lutgemm_weight *c : copies) {
+            if (rows > kTableRows) {
+                c->plan_batch[rows > 8] = p;
+                c->batch_measured[rows > 8] = true;
+            } else {
+                (rows == 2 ? c->plan2 : c->plan) = p;
+            }
+        }
         int stt = LUTGEMM_OK;
         for (int r = 0; r < 2 && stt == LUTGEMM_OK; r++)
             stt = run_matvec(copies[turn++ % copies.size()], x, y, rows, stream, false, false);
@@ -1032,8 +1069,48 @@ int lutgemm_weight_autotune(lutgemm_weight *w, void *stream)
                 }
             }
     }
+    // The batch kernel, for passes of up to 8 rows and of 9..16 rows: the model's ten best plans,
+    // measured the same way.
+    Plan chosen_batch[2] = {before_batch[0], before_batch[1]};
+    bool have_batch[2] = {false, false};
+    for (int bi = 0; bi < 2 && batch_kernel_takes(s); bi++) {
+        const int rows = bi ? kRowsPerPass : 8;
+        struct Timed { float ms; double cost; Plan p; };
+        std::vector<Timed> timed;
+        for (int waves = lutgemm_kernels::batch_waves_min(rows); waves <= lutgemm_kernels::kBatchWaves; waves++)
+            for (int ks = 1; ks <= s.ts && ks <= kMaxSplits; ks++) {
+                Plan p;
+                const double cost = batch_plan_cost(s, w->compute_units, waves, ks, &p);
+                if (cost >= 0.0) timed.push_back(Timed{1e30f, cost, p});
+            }
+        std::sort(timed.begin(), timed.end(), [](const Timed &a, const Timed &b) { return a.cost < b.cost; });
+        if (timed.size() > 10) timed.resize(10);
+        for (int sweep = 0; sweep < 2; sweep++)
+            for (size_t i = 0; status == LUTGEMM_OK && i < timed.size(); i++) {
+                float ms = 0.f;
+                status = measure(timed[i].p, rows, 8, &ms);
+                if (status == LUTGEMM_OK && ms < timed[i].ms) timed[i].ms = ms;
+            }
+        std::sort(timed.begin(), timed.end(), [](const Timed &a, const Timed &b) { return a.ms < b.ms; });
+        float best_ms = 1e30f;
+        for (int round = 0; round < 2; round++)
+            for (size_t i = 0; status == LUTGEMM_OK && i < timed.size() && i < 3; i++) {
+                float ms = 0.f;
+                status = measure(timed[i].p, rows, 30, &ms);
+                if (status == LUTGEMM_OK && ms < best_ms) {
+                    best_ms = ms;
+                    chosen_batch[bi] = timed[i].p;
+                    have_batch[bi] = true;
+                }
+            }
+    }
     w->plan = status == LUTGEMM_OK ? chosen[0] : before;
     w->plan2 = status == LUTGEMM_OK ? chosen[1] : before2;
+    for (int bi = 0; bi < 2; bi++) {
+        const bool ok = status == LUTGEMM_OK && have_batch[bi];
+        w->plan_batch[bi] = ok ? chosen_batch[bi] : before_batch[bi];
+        w->batch_measured[bi] = ok ? true : before_measured[bi];
+    }
     if (e0) (void)hipEventDestroy(e0);
     if (e1) (void)hipEventDestroy(e1);
     if (x) (void)hipFree(x);

@@ -245,18 +245,20 @@ def test_autotune_keeps_results_and_picks_a_valid_plan(lutgemm, oracle, device):
     from lutgemm import synth
     k, n, q, g = 4096, 2048, 3, 128
     w, W = make(lutgemm, synth, k, n, q, g, offset=True, seed=21)
-    x = synth.make_x(5, k, seed=21)
+    x = synth.make_x(12, k, seed=21)
     truth = truth_of(oracle, w, x)
     say("case autotune")
     plan = W.autotune(torch.cuda.current_stream().cuda_stream)
     assert 1 <= plan["waves"] <= 12 and 1 <= plan["k_splits"] <= 8
     assert plan["workgroups"] == -(-(n // 32) // plan["waves"]) * plan["k_splits"]
     singles = np.concatenate([run_matvec(lutgemm, W, x[r:r + 1], device) for r in range(5)])
-    assert_within_tolerance(singles, truth, "after autotune %s" % plan)
+    assert_within_tolerance(singles, truth[:5], "after autotune %s" % plan)
     # two-row passes keep a measured plan of their own; their rows must still equal the one-row launches
     y = run_matvec(lutgemm, W, x[:2], device)
     assert np.array_equal(y.view(np.uint16), singles[:2].view(np.uint16))
-    for m in (3, 5):   # the batch kernel: another order of additions, same tolerance
+    # the batch kernel (measured plans for passes of up to 8 and of 9..16 rows): another order
+    # of additions, same tolerance
+    for m in (3, 5, 12):
         assert_within_tolerance(run_matvec(lutgemm, W, x[:m], device), truth[:m], "m=%d" % m)
     W.close()
 
