@@ -56,7 +56,7 @@ typedef __attribute__((address_space(3))) unsigned char lds_byte;
 constexpr int kPatternBytes = 256 * 16 * 16;               // 64 KiB: [pattern][lane slot][16 bytes]
 constexpr int kXRowBytes = kBlockK * 2 + 16;               // one activation row of a k-block, padded:
                                                            // 16 rows read at one column hit 64 different banks
-constexpr int kXBufBytes = kBatchRows * kXRowBytes;        // 16,640
+constexpr int kXBufBytes = (kBatchRows + 1) * kXRowBytes;  // 17,680: 16 rows and a spare one that is never read
 constexpr int kStageBytes = 1024;                          // per wavefront: [16 outputs][64 chunk positions]
 constexpr int kScaleAreaBytes = 256 * 5;                   // per wavefront: up to 5 scale words of its 64 lanes, [word][lane]
 
@@ -65,21 +65,22 @@ __host__ __device__ constexpr int batch_lds_bytes(int waves)
     return kPatternBytes + 2 * kXBufBytes + waves * (kStageBytes + kScaleAreaBytes);
 }
 
-// The activation block of k-block ts is 16 rows x 64 chunks of 16 bytes.  Wavefront w moves row w
-// (the launch has at least as many wavefronts as the batch has rows), lane = chunk.  The load and
-// the LDS write are separate so that the load of the next block is in flight while the current
-// one is processed.  k beyond the weight reads as zero; rows beyond the batch are never written
-// and keep the zeros the buffers start with.  No branches: a branch in the loop body costs the
-// register allocator dearly, and with straight-line code the wait counts of the loads stay exact.
-__device__ __forceinline__ u32x4 load_activation_row(const MatvecArgs &a, int ts, int wave, int lane, bool valid)
+// The activation block of k-block ts is 16 rows x 64 chunks of 16 bytes.  Wavefront w moves rows w
+// and w + waves (a launch has at least 8 wavefronts, so two rows per wavefront cover the 16 of a
+// pass), lane = chunk.  The load and the LDS write are separate so that the load of the next block
+// is in flight while the current one is processed.  k beyond the weight and rows beyond the batch
+// read as zero.  No branches: a
+// branch in the loop body costs the register allocator dearly, and with straight-line code the
+// wait counts of the loads stay exact.
+__device__ __forceinline__ u32x4 load_activation_row(const MatvecArgs &a, int ts, int row, int lane, bool valid)
 {
     const __half *x = reinterpret_cast<const __half *>(a.x);
     // A row is kept in LDS ordered [kappa = chunk % 4][t = chunk / 4]: position L holds chunk
     // 4 (L % 16) + L / 16, so that the 16-byte reads of the matrix lanes (kappa, j) at step t fall
     // into bank groups that depend on j and t only (see the read in the kernel).
     const int kpos = ts * kBlockK + (4 * (lane & 15) + (lane >> 4)) * kChunk;
-    const uint32_t m = 0u - (uint32_t)(valid && wave < a.rows && kpos < a.k);
-    const size_t offset = ((size_t)wave * (size_t)a.x_row_stride + (size_t)kpos) & (size_t)(0 - (long long)(m & 1u));
+    const uint32_t m = 0u - (uint32_t)(valid && row < a.rows && kpos < a.k);
+    const size_t offset = ((size_t)row * (size_t)a.x_row_stride + (size_t)kpos) & (size_t)(0 - (long long)(m & 1u));
     u32x4 v = *reinterpret_cast<const u32x4 *>(x + offset);
     v.x &= m;
     v.y &= m;
@@ -88,9 +89,12 @@ __device__ __forceinline__ u32x4 load_activation_row(const MatvecArgs &a, int ts
     return v;
 }
 
-__device__ __forceinline__ void store_activation_row(const u32x4 &v, lds_byte *buf, int wave, int lane)
+__device__ __forceinline__ void store_activation_row(const u32x4 &v, lds_byte *buf, int row, int lane)
 {
-    *reinterpret_cast<__attribute__((address_space(3))) u32x4 *>(buf + wave * kXRowBytes + lane * 16) = v;
+    // rows 16 and up (second rows of the wavefronts of a large workgroup) do not exist: their zeros
+    // go to a spare row behind the 16, so that the store needs no branch
+    const int slot = row < kBatchRows ? row : kBatchRows;
+    *reinterpret_cast<__attribute__((address_space(3))) u32x4 *>(buf + slot * kXRowBytes + lane * 16) = v;
 }
 
 // LDS reads whose order and wait counts are fixed by hand.  The compiler waits for every LDS read
@@ -130,9 +134,11 @@ __device__ __forceinline__ void after_wait(half8 &v) { asm volatile("" : "+v"(v)
 __device__ __forceinline__ void after_wait(uint32_t &v) { asm volatile("" : "+v"(v)); }
 
 // W is the largest number of wavefronts a workgroup may have (it sets the register budget); the
-// launch picks a number up to it (and not below the rows of the batch) that divides the column
-// batches of the shape well over the compute units.
-template <int Q, bool OFF, int W>
+// launch picks a number from eight up to it that divides the column batches of the shape well
+// over the compute units.  TWO: the batch has more rows than the workgroup has wavefronts, so
+// every wavefront stages a second activation row (a build of its own: the second row's load and
+// store cost the batches that do not need them 2.5 %).
+template <int Q, bool OFF, int W, bool TWO>
 __global__ __launch_bounds__(W * 64) void lut_batch_kernel(MatvecArgs a)
 {
     constexpr int QO = Q + (OFF ? 1 : 0);
@@ -193,8 +199,11 @@ __global__ __launch_bounds__(W * 64) void lut_batch_kernel(MatvecArgs a)
     for (int idx = tid; idx < 2 * kXBufBytes / 16; idx += threads)
         *reinterpret_cast<__attribute__((address_space(3))) u32x4 *>(xbuf + idx * 16) = u32x4{0u, 0u, 0u, 0u};
     u32x4 xrow = load_activation_row(a, ts0, wave, lane, true);
+    u32x4 xrow2 = u32x4{0u, 0u, 0u, 0u};
+    if constexpr (TWO) xrow2 = load_activation_row(a, ts0, wave + waves, lane, true);
     __syncthreads();   // the zeros are in place before the first rows go on top of them
     store_activation_row(xrow, xbuf, wave, lane);
+    if constexpr (TWO) store_activation_row(xrow2, xbuf, wave + waves, lane);
 
 
     // lane roles
@@ -240,6 +249,7 @@ __global__ __launch_bounds__(W * 64) void lut_batch_kernel(MatvecArgs a)
         const bool more = ts + 1 < ts1;
         const NextTile next = tile_address<Q, QO, 1>(signs, scales, tile0 + ts + 1, lane, more);
         xrow = load_activation_row(a, ts + 1, wave, lane, more);
+        if constexpr (TWO) xrow2 = load_activation_row(a, ts + 1, wave + waves, lane, more);
 
         // this k-block's scale words into the wavefront's LDS area, then the refill of their registers
 #pragma unroll
@@ -393,6 +403,7 @@ __global__ __launch_bounds__(W * 64) void lut_batch_kernel(MatvecArgs a)
             });
         }
         store_activation_row(xrow, xbuf + (cur ^ 1) * kXBufBytes, wave, lane);
+        if constexpr (TWO) store_activation_row(xrow2, xbuf + (cur ^ 1) * kXBufBytes, wave + waves, lane);
         __syncthreads();   // the next activation block is in place; this one is no longer read
     }
 
@@ -430,7 +441,7 @@ __global__ __launch_bounds__(W * 64) void lut_batch_kernel(MatvecArgs a)
         for (int v = 0; v < 4; v++) complete_output(arrival[h][v], valid[h][v], word[h][v], yout[h][v], a.k_splits);
 }
 
-template <int Q, bool OFF, int W>
+template <int Q, bool OFF, int W, bool TWO>
 hipError_t launch_batch_w(const MatvecArgs &a, int workgroups, int waves, hipStream_t stream)
 {
     static std::atomic<unsigned long long> allowed{0};
@@ -439,12 +450,12 @@ hipError_t launch_batch_w(const MatvecArgs &a, int workgroups, int waves, hipStr
     if (e != hipSuccess) return e;
     const unsigned long long bit = 1ull << (dev & 63);
     if (!(allowed.load(std::memory_order_relaxed) & bit)) {
-        e = hipFuncSetAttribute(reinterpret_cast<const void *>(&lut_batch_kernel<Q, OFF, W>),
+        e = hipFuncSetAttribute(reinterpret_cast<const void *>(&lut_batch_kernel<Q, OFF, W, TWO>),
                                 hipFuncAttributeMaxDynamicSharedMemorySize, batch_lds_bytes(W));
         if (e != hipSuccess) return e;
         allowed.fetch_or(bit, std::memory_order_relaxed);
     }
-    hipLaunchKernelGGL((lut_batch_kernel<Q, OFF, W>), dim3(workgroups), dim3(waves * kLanes), batch_lds_bytes(waves), stream,
+    hipLaunchKernelGGL((lut_batch_kernel<Q, OFF, W, TWO>), dim3(workgroups), dim3(waves * kLanes), batch_lds_bytes(waves), stream,
                        a);
     return hipGetLastError();
 }
@@ -453,8 +464,10 @@ template <int Q>
 hipError_t launch_batch_off(int has_offset, const MatvecArgs &a, int wg, int waves, hipStream_t s)
 {
     constexpr int W = kBatchWaves;
-    if (waves < batch_waves_min(a.rows) || waves > W) return hipErrorInvalidValue;
-    return has_offset ? launch_batch_w<Q, true, W>(a, wg, waves, s) : launch_batch_w<Q, false, W>(a, wg, waves, s);
+    if (waves < kBatchWavesMin || waves > W) return hipErrorInvalidValue;
+    if (a.rows > waves)
+        return has_offset ? launch_batch_w<Q, true, W, true>(a, wg, waves, s) : launch_batch_w<Q, false, W, true>(a, wg, waves, s);
+    return has_offset ? launch_batch_w<Q, true, W, false>(a, wg, waves, s) : launch_batch_w<Q, false, W, false>(a, wg, waves, s);
 }
 
 }  // namespace

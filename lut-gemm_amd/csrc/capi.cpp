@@ -206,9 +206,9 @@ double batch_plan_cost(const Shape &s, int cus, int waves, int ks, Plan *out)
     return rounds * (bps * (waves * tile_us + block_us) + start_us) + (rounds - 1) * round_us + 0.02 * ks;
 }
 
-Plan choose_batch_plan(const Shape &s, int rows, int cus)
+Plan choose_batch_plan(const Shape &s, int cus)
 {
-    const int wmax = lutgemm_kernels::kBatchWaves, wmin = lutgemm_kernels::batch_waves_min(rows);
+    const int wmax = lutgemm_kernels::kBatchWaves, wmin = lutgemm_kernels::kBatchWavesMin;
     Plan best{wmax, div_up(s.nb, wmax), s.ts, 1};
     double best_cost = 1e30;
     long best_wgs = 0;
@@ -520,7 +520,7 @@ int run_matvec(const lutgemm_weight *w, const void *x, void *y, int m, void *str
         // up to 16 rows per pass over the weight on the matrix cores
         const int pass_rows = m < kRowsPerPass ? m : kRowsPerPass;
         const Plan plan = w->batch_measured[pass_rows > 8] ? w->plan_batch[pass_rows > 8]
-                                                            : choose_batch_plan(s, pass_rows, w->compute_units);
+                                                            : choose_batch_plan(s, w->compute_units);
         a.ntiles = plan.ntiles;
         a.k_splits = plan.k_splits;
         a.blocks_per_split = plan.blocks_per_split;
@@ -1077,7 +1077,7 @@ int lutgemm_weight_autotune(lutgemm_weight *w, void *stream)
         const int rows = bi ? kRowsPerPass : 8;
         struct Timed { float ms; double cost; Plan p; };
         std::vector<Timed> timed;
-        for (int waves = lutgemm_kernels::batch_waves_min(rows); waves <= lutgemm_kernels::kBatchWaves; waves++)
+        for (int waves = lutgemm_kernels::kBatchWavesMin; waves <= lutgemm_kernels::kBatchWaves; waves++)
             for (int ks = 1; ks <= s.ts && ks <= kMaxSplits; ks++) {
                 Plan p;
                 const double cost = batch_plan_cost(s, w->compute_units, waves, ks, &p);

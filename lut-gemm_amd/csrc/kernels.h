@@ -57,11 +57,11 @@ hipError_t launch_matvec_multi(int q, int has_offset, int gsub, const MultiMatve
                                hipStream_t stream);
 
 // 1..kBatchRows activation rows in one pass (matrix cores); scale layouts with gsub == 1 and up to
-// kBatchMaxPlanes planes only.  A workgroup has batch_waves_min(rows) .. kBatchWaves wavefronts:
-// wavefront w stages activation row w, so there are at least as many as the batch has rows.
+// kBatchMaxPlanes planes only.  A workgroup has kBatchWavesMin .. kBatchWaves wavefronts:
+// wavefront w stages activation rows w and w + wavefronts, so eight cover the 16 rows of a pass.
 constexpr int kBatchMaxPlanes = 4;
 constexpr int kBatchWaves = 16;
-constexpr int batch_waves_min(int rows) { return rows > 8 ? rows : 8; }
+constexpr int kBatchWavesMin = 8;
 hipError_t launch_batch(int q, int has_offset, const MatvecArgs &a, int workgroups, int waves, hipStream_t stream);
 
 // words[0..count) = 0 (a fill kernel rather than a memset node, so that it can be captured)
