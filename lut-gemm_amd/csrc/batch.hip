@@ -177,7 +177,7 @@ __global__ __launch_bounds__(W * 64) void lut_batch_kernel(MatvecArgs a)
     u32x4 sign[NU];
     uint32_t scale[QO];
     {
-        const NextTile n0 = tile_address<Q, QO, 1>(signs, scales, tile0 + ts0, lane, true);
+        const NextTile n0 = tile_address_uniform<Q, QO, 1>(signs, scales, tile0 + ts0, lane, true);
 #pragma unroll
         for (int d = 0; d < QO; d++) scale[d] = __builtin_nontemporal_load(n0.scale + d);
 #pragma unroll
@@ -247,7 +247,7 @@ __global__ __launch_bounds__(W * 64) void lut_batch_kernel(MatvecArgs a)
     for (int ts = ts0; ts < ts1; ts++) {
         const int cur = (ts - ts0) & 1;
         const bool more = ts + 1 < ts1;
-        const NextTile next = tile_address<Q, QO, 1>(signs, scales, tile0 + ts + 1, lane, more);
+        const NextTile next = tile_address_uniform<Q, QO, 1>(signs, scales, tile0 + ts + 1, lane, more);
         xrow = load_activation_row(a, ts + 1, wave, lane, more);
         if constexpr (TWO) xrow2 = load_activation_row(a, ts + 1, wave + waves, lane, more);
 

@@ -43,6 +43,22 @@ __device__ __forceinline__ NextTile tile_address(const u32x4 *signs, const uint3
     return n;
 }
 
+// The same for a kernel that can afford a whole tile of loads past the end of its range: the tile
+// number becomes 0 there (tile 0 stays in the cache: every workgroup ends on it).  `tile` and
+// `real` are wave-uniform, so an address is a uniform base plus a lane constant plus an immediate
+// and the address arithmetic stays on the scalar unit.
+template <int Q, int QO, int GSUB>
+__device__ __forceinline__ NextTile tile_address_uniform(const u32x4 *signs, const uint32_t *scales, size_t tile,
+                                                         int lane, bool real)
+{
+    const size_t t = real ? tile : (size_t)0;
+    NextTile n;
+    n.scale = scales + t * (size_t)(kLanes * GSUB * QO) + lane * (GSUB * QO);
+    n.sign = signs + t * (size_t)(2 * Q * kLanes) + lane;
+    n.sign_stride = (size_t)kLanes;
+    return n;
+}
+
 template <int Q, int QO, int GSUB>
 __device__ __forceinline__ void load_tile(TileRegs<Q, QO, GSUB> &r, const NextTile &n)
 {
