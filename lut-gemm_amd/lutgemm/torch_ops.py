@@ -8,10 +8,23 @@ be captured into a HIP graph like any other torch op.  Batches larger than `dens
 rows go through the dequantised fp16 weight and the library GEMM, the route the reference takes
 for every m > 1 (lutGEMM/src/kernels.cu:73-79); up to it the library streams the packed weight
 (one or two rows through the table-lookup kernels, more through the batch kernel, 16 rows per
-pass).  The default threshold is where two passes of the batch kernel meet a library GEMM over
-the dense weight on MI355X (about 32 rows at k = n = 12288).
+pass).  The default threshold depends on the weight (default_dense_threshold): it is where the
+two routes met when measured on MI355X.
 """
-DENSE_THRESHOLD = 32
+
+
+def default_dense_threshold(weight):
+    """Rows up to which the packed routes beat dequantised weight + library GEMM (measured on
+    MI355X at k = n = 12288 and k = 12288, n = 49152; LutLinear(dense_threshold=...) overrides).
+
+    Shapes the batch kernel takes (group size a multiple of 128, up to four planes): one pass of
+    16 rows costs 21-37 us against 50 us for the GEMM, two passes 40-72 us against 56 us: 32 rows
+    for one or two planes, 16 for three or four.  Other shapes go through two-row passes of the
+    table-lookup kernel, which lose to the GEMM from three rows on."""
+    if weight.group_size % 128 == 0 and weight.nb <= 4:
+        return 32 if weight.nb <= 2 else 16
+    return 2
+
 
 import weakref
 
@@ -69,7 +82,7 @@ class LutLinear(torch.nn.Module):
     container: dict(bW, alpha, q_bias, k, n, q, num_groups) as quantize.to_container returns.
     """
 
-    def __init__(self, container, bias=None, dense_threshold=DENSE_THRESHOLD, autotune=False):
+    def __init__(self, container, bias=None, dense_threshold=None, autotune=False):
         super().__init__()
         c = container
         self.weight = BCQWeight(c["bW"], c["alpha"], c["k"], c["n"], c["q"], c["num_groups"], c.get("q_bias"))
@@ -77,7 +90,7 @@ class LutLinear(torch.nn.Module):
             self.weight.autotune(torch.cuda.current_stream().cuda_stream)
         self.handle = register(self.weight)
         self.in_features, self.out_features = c["k"], c["n"]
-        self.dense_threshold = dense_threshold
+        self.dense_threshold = default_dense_threshold(self.weight) if dense_threshold is None else dense_threshold
         self._dense = None
         if bias is not None:
             self.register_buffer("bias", torch.as_tensor(bias).to(torch.float16).cuda())
@@ -93,7 +106,8 @@ class LutLinear(torch.nn.Module):
             self.weight.autotune(torch.cuda.current_stream().cuda_stream)
         self.handle = register(self.weight)
         self.in_features, self.out_features = self.weight.kSize, self.weight.mSize
-        self.dense_threshold = kw.get("dense_threshold", DENSE_THRESHOLD)
+        dt = kw.get("dense_threshold")
+        self.dense_threshold = default_dense_threshold(self.weight) if dt is None else dt
         self._dense = None
         if bias is not None:
             self.register_buffer("bias", torch.as_tensor(bias).to(torch.float16).cuda())

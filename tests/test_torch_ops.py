@@ -95,3 +95,17 @@ def test_operator_argument_checks(lutgemm, device):
         torch.ops.lutgemm.matvec(torch.zeros(1, 512, dtype=torch.float16, device=device), layer.handle)
     with pytest.raises(Exception):
         torch.ops.lutgemm.matvec(torch.zeros(1, 1024, dtype=torch.float16, device=device), 10 ** 9)
+
+
+def test_default_dense_threshold_follows_the_weight(lutgemm, device):
+    """Shapes the batch kernel takes keep the packed route for one or two passes of 16 rows,
+    every other shape leaves it from three rows on."""
+    from lutgemm import quantize, torch_ops
+    print("case default dense threshold", flush=True)
+    lin, _ = _layer(5, out_f=64, in_f=512, bias=False)
+    for qbits, g, want in ((2, 128, 32), (4, 128, 16), (3, 64, 2), (5, 128, 2)):
+        c, _ = quantize.quantize_linear(lin.weight.detach(), qbits, g, "rtn", rounds=0)
+        layer = torch_ops.LutLinear(c)
+        assert layer.dense_threshold == want, (qbits, g, layer.dense_threshold)
+        assert torch_ops.LutLinear(c, dense_threshold=7).dense_threshold == 7
+        layer.weight.close()
