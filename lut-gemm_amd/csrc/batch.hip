@@ -27,8 +27,8 @@
 //    Products of fp16 numbers are exact in fp32, so the only roundings are fp32 additions.
 //  * At the end every (row, output) goes through the same split-k completion as the one-row kernel.
 //
-// Only scale layouts with one group per 128 k (group size a multiple of 128) are handled here;
-// other group sizes keep the two-row table kernel.
+// Scale groups of 128 k and more are applied once per four MFMAs; groups of 64 or 32 k (two or
+// four per 128 k) after two or after every MFMA, with the scales re-ordered through LDS first.
 #include <hip/hip_fp16.h>
 #include <hip/hip_runtime.h>
 
@@ -57,14 +57,8 @@ constexpr int kPatternBytes = 256 * 16 * 16;               // 64 KiB: [pattern][
 constexpr int kXRowBytes = kBlockK * 2 + 16;               // one activation row of a k-block, padded:
                                                            // 16 rows read at one column hit 64 different banks
 constexpr int kXBufBytes = (kBatchRows + 1) * kXRowBytes;  // 17,680: 16 rows and a spare one that is never read
+static_assert(batch_lds_bytes(0, 1, 1) == kPatternBytes + 2 * kXBufBytes, "kernels.h states the LDS of this kernel");
 constexpr int kStageBytes = 1024;                          // per wavefront: [16 outputs][64 chunk positions]
-constexpr int kScaleAreaBytes = 256 * 5;                   // per wavefront: up to 5 scale words of its 64 lanes, [word][lane]
-
-__host__ __device__ constexpr int batch_lds_bytes(int waves)
-{
-    return kPatternBytes + 2 * kXBufBytes + waves * (kStageBytes + kScaleAreaBytes);
-}
-
 // The activation block of k-block ts is 16 rows x 64 chunks of 16 bytes.  Wavefront w moves rows w
 // and w + waves (a launch has at least 8 wavefronts, so two rows per wavefront cover the 16 of a
 // pass), lane = chunk.  The load and the LDS write are separate so that the load of the next block
@@ -138,10 +132,13 @@ __device__ __forceinline__ void after_wait(uint32_t &v) { asm volatile("" : "+v"
 // over the compute units.  TWO: the batch has more rows than the workgroup has wavefronts, so
 // every wavefront stages a second activation row (a build of its own: the second row's load and
 // store cost the batches that do not need them 2.5 %).
-template <int Q, bool OFF, int W, bool TWO>
+template <int Q, bool OFF, int GSUB, int W, bool TWO>
 __global__ __launch_bounds__(W * 64) void lut_batch_kernel(MatvecArgs a)
 {
     constexpr int QO = Q + (OFF ? 1 : 0);
+    constexpr int SW = GSUB * QO;   // scale words a lane holds per tile
+    constexpr int SG = 4 / GSUB;    // matrix instructions per scale group (a k-block has 4 GSUB groups)
+    constexpr int SUBL = 16 / GSUB; // lanes of a row that share a scale group
     constexpr int NU = 2 * Q;   // sign vectors (units) of a tile: unit U = plane U / 2, output half U % 2
     constexpr int CH = NU <= 6 ? NU : NU % 6 == 0 ? 6 : NU % 5 == 0 ? 5 : NU % 4 == 0 ? 4 : 2;   // units per pass
     constexpr int P = Q <= 2 ? LUTGEMM_BATCH_AHEAD : 0;   // steps of LDS reads in flight ahead of the matrix instructions (0: the compiler's order)
@@ -163,7 +160,7 @@ __global__ __launch_bounds__(W * 64) void lut_batch_kernel(MatvecArgs a)
     const bool active = nb < a.nb;
     const int ts0 = ks * a.blocks_per_split;
     const int ts1 = min(ts0 + a.blocks_per_split, a.ts);
-    lds_byte *stage = lds + kPatternBytes + 2 * kXBufBytes + wave * (kStageBytes + kScaleAreaBytes);
+    lds_byte *stage = lds + kPatternBytes + 2 * kXBufBytes + wave * (kStageBytes + batch_scale_area_bytes(GSUB, QO));
     lds_byte *scale_area = stage + kStageBytes;
 
     const u32x4 *signs = reinterpret_cast<const u32x4 *>(a.signs);
@@ -175,11 +172,11 @@ __global__ __launch_bounds__(W * 64) void lut_batch_kernel(MatvecArgs a)
     // groups of the k-block for their two outputs (j and 16 + j); group r is held by lane 16 r + j,
     // so every wavefront passes its scale words through a small LDS area of its own, [word][lane].
     u32x4 sign[NU];
-    uint32_t scale[QO];
+    uint32_t scale[SW];
     {
-        const NextTile n0 = tile_address_uniform<Q, QO, 1>(signs, scales, tile0 + ts0, lane, true);
+        const NextTile n0 = tile_address_uniform<Q, QO, GSUB>(signs, scales, tile0 + ts0, lane, true);
 #pragma unroll
-        for (int d = 0; d < QO; d++) scale[d] = __builtin_nontemporal_load(n0.scale + d);
+        for (int d = 0; d < SW; d++) scale[d] = __builtin_nontemporal_load(n0.scale + d);
 #pragma unroll
         for (int u = 0; u < NU; u++) sign[u] = __builtin_nontemporal_load(n0.sign + u * n0.sign_stride);
     }
@@ -232,10 +229,32 @@ __global__ __launch_bounds__(W * 64) void lut_batch_kernel(MatvecArgs a)
     // bytes 0, 2 and 3 of a pattern address: lane slot and the LDS address bits above 64 KiB
     const uint32_t pattern_lane = ((uint32_t)j << 4) + (uint32_t)(size_t)pattern;
 
+    // One group per 128 k: the scale words go to LDS as they are, [word][lane]; the matrix lane
+    // (kappa, j) finds the pair (output j, output 16 + j) of 128-k group r at lane 16 r + j.
+    // Two or four groups per 128 k: lane (row r, sub-row sub, jj) holds, in slot t, the scales of
+    // output t SUBL + jj for the group (r, sub); each fp16 number goes to
+    // [group r GSUB + sub][plane or offset][output % 16][output / 16], so that the matrix lanes
+    // again read one word per (group, plane) with the pair (output j, output 16 + j).
     __attribute__((address_space(3))) uint32_t *scale_w =
         reinterpret_cast<__attribute__((address_space(3))) uint32_t *>(scale_area) + lane;
+    // (the halves are read back as 32-bit words: the write type may alias them)
+    typedef uint16_t __attribute__((may_alias)) aliasing_u16;
+    __attribute__((address_space(3))) aliasing_u16 *scale_wh = reinterpret_cast<__attribute__((address_space(3))) aliasing_u16 *>(
+        scale_area + ((((lane >> 4) * GSUB + (lane & 15) / SUBL) * QO) * 16 + (lane & 15) % SUBL) * 4);
     const __attribute__((address_space(3))) uint32_t *scale_r =
         reinterpret_cast<const __attribute__((address_space(3))) uint32_t *>(scale_area) + j;
+    // LDS byte offset (from scale_r) of the word of scale group G (0 .. 4 GSUB - 1 of the k-block) that
+    // holds fp16 number hb = half * QO + plane-or-offset (GSUB 1) or the pair of plane-or-offset b
+    auto scale_word_offset = [](int G, int idx) constexpr {
+        return GSUB == 1 ? (idx * kLanes + 16 * G) * 4 : ((G * QO + idx) * 16) * 4;
+    };
+    // the fp16 number of (plane or offset b, output half h) out of the words of one group
+    auto scale_value = [](const uint32_t (&words)[QO], int b, int h) {
+        const int hb = h * QO + b;
+        const uint32_t w = GSUB == 1 ? words[hb >> 1] : words[b];
+        const __half2 h2 = *reinterpret_cast<const __half2 *>(&w);
+        return (GSUB == 1 ? (hb & 1) : h) ? __high2float(h2) : __low2float(h2);
+    };
 
     float4v acc[2];
     acc[0] = float4v{0.f, 0.f, 0.f, 0.f};
@@ -247,20 +266,32 @@ __global__ __launch_bounds__(W * 64) void lut_batch_kernel(MatvecArgs a)
     for (int ts = ts0; ts < ts1; ts++) {
         const int cur = (ts - ts0) & 1;
         const bool more = ts + 1 < ts1;
-        const NextTile next = tile_address_uniform<Q, QO, 1>(signs, scales, tile0 + ts + 1, lane, more);
+        const NextTile next = tile_address_uniform<Q, QO, GSUB>(signs, scales, tile0 + ts + 1, lane, more);
         xrow = load_activation_row(a, ts + 1, wave, lane, more);
         if constexpr (TWO) xrow2 = load_activation_row(a, ts + 1, wave + waves, lane, more);
 
         // this k-block's scale words into the wavefront's LDS area, then the refill of their registers
+        if constexpr (GSUB == 1) {
 #pragma unroll
-        for (int d = 0; d < QO; d++) scale_w[d * kLanes] = scale[d];
+            for (int d = 0; d < SW; d++) scale_w[d * kLanes] = scale[d];
+        } else {
+            static_for<2 * SW>([&](auto F) {
+                constexpr int f = F, t = f / QO, bo = f % QO;   // slot t: output t SUBL + jj
+                constexpr int dest = (bo * 16 + (t % GSUB) * SUBL) * 2 + t / GSUB;   // in fp16 units from scale_wh
+                scale_wh[dest] = (uint16_t)(scale[f >> 1] >> (16 * (f & 1)));
+            });
+        }
+        // the reads of these words further down are asm statements or reads through another pointer
+        // type: keep the compiler from moving them above the writes (no instruction is emitted)
+        asm volatile("" ::: "memory");
 #pragma unroll
-        for (int d = 0; d < QO; d++) scale[d] = __builtin_nontemporal_load(next.scale + d);
-        // fp16 number hb (= output half * QO + plane-or-offset) of group r as fp32
-        auto scale_of = [&](int r, int hb) {
-            const uint32_t w = scale_r[(hb >> 1) * kLanes + 16 * r];
+        for (int d = 0; d < SW; d++) scale[d] = __builtin_nontemporal_load(next.scale + d);
+        // the words of scale group G, read when needed (the paths without hand-placed reads)
+        auto scale_of = [&](int G, int b, int h) {
+            const int hb = h * QO + b;
+            const uint32_t w = scale_r[scale_word_offset(G, GSUB == 1 ? hb >> 1 : b) / 4];
             const __half2 h2 = *reinterpret_cast<const __half2 *>(&w);
-            return (hb & 1) ? __high2float(h2) : __low2float(h2);
+            return (GSUB == 1 ? (hb & 1) : h) ? __high2float(h2) : __low2float(h2);
         };
 
         const lds_byte *xr = xbuf + cur * kXBufBytes + j * kXRowBytes + kappa * 256;
@@ -281,7 +312,7 @@ __global__ __launch_bounds__(W * 64) void lut_batch_kernel(MatvecArgs a)
                 sign[U] = __builtin_nontemporal_load(next.sign + U * next.sign_stride);
             });
             if constexpr (P > 0) {
-                // Steps g = 0..15 of the k-block (MFMA t = g: group g / 4): the LDS reads of step
+                // Steps g = 0..15 of the k-block (MFMA t = g: scale group g / SG): the LDS reads of step
                 // g + P are issued before step g is waited for and contracted.
                 half8 xa[P + 1];
                 half8 bits[P + 1][CH];
@@ -297,16 +328,17 @@ __global__ __launch_bounds__(W * 64) void lut_batch_kernel(MatvecArgs a)
                         constexpr uint32_t sel = 0x03020400u + ((uint32_t)(g & 3) << 8);   // address byte 1 <- sign byte g % 4
                         bits[slot][I] = lds_read128(__builtin_amdgcn_perm(word, pattern_lane, sel));
                     });
-                    if constexpr ((g & 3) == 3)
-                        static_for<QO>([&](auto Wd) { sw[(g >> 2) & 1][Wd] = lds_read32_at<(Wd * kLanes + 16 * (g >> 2)) * 4>(saddr); });
+                    if constexpr (g % SG == SG - 1)
+                        static_for<QO>([&](auto Wd) { sw[(g / SG) & 1][Wd] = lds_read32_at<scale_word_offset(g / SG, Wd)>(saddr); });
                 };
                 static_for<P>(issue);
                 static_for<16>([&](auto Gc) {
-                    constexpr int g = Gc, r = g >> 2, TT = g & 3, slot = g % (P + 1);
+                    constexpr int g = Gc, G = g / SG, TT = g % SG, slot = g % (P + 1);
                     if constexpr (g + P < 16) issue(std::integral_constant<int, (g + P < 16 ? g + P : 0)>{});
                     // reads younger than those of step g: the steps g + 1 .. g + P that exist
                     constexpr int last = g + P < 16 ? g + P : 15;
-                    constexpr int younger = (last - g) * (1 + CH) + QO * ((last >> 2) - (g >> 2) + ((last & 3) == 3) - ((g & 3) == 3));
+                    // (the scale words of a group are read with its last step: (x + 1) / SG groups end by step x)
+                    constexpr int younger = (last - g) * (1 + CH) + QO * ((last + 1) / SG - (g + 1) / SG);
                     lds_wait<younger>(xa[slot]);
                     static_for<CH>([&](auto I) {
                         after_wait(bits[slot][I]);
@@ -315,16 +347,11 @@ __global__ __launch_bounds__(W * 64) void lut_batch_kernel(MatvecArgs a)
                     if constexpr (OFF)
                         xsum = __builtin_amdgcn_mfma_f32_16x16x32_f16(xa[slot], __builtin_bit_cast(half8, ones),
                                                                       TT == 0 ? zero4 : xsum, 0, 0, 0);
-                    if constexpr (TT == 3) {
-                        static_for<QO>([&](auto Wd) { after_wait(sw[r & 1][Wd]); });
-                        auto scale_word = [&](int hb) {
-                            const uint32_t w = sw[r & 1][hb >> 1];
-                            const __half2 h2 = *reinterpret_cast<const __half2 *>(&w);
-                            return (hb & 1) ? __high2float(h2) : __low2float(h2);
-                        };
+                    if constexpr (TT == SG - 1) {
+                        static_for<QO>([&](auto Wd) { after_wait(sw[G & 1][Wd]); });
                         static_for<CH>([&](auto I) {
                             constexpr int U = u0 + I, b = U / 2, h = U % 2;
-                            const float sc = scale_word(h * QO + b);
+                            const float sc = scale_value(sw[G & 1], b, h);
                             acc[h][0] += sc * part[I][0];
                             acc[h][1] += sc * part[I][1];
                             acc[h][2] += sc * part[I][2];
@@ -333,7 +360,7 @@ __global__ __launch_bounds__(W * 64) void lut_batch_kernel(MatvecArgs a)
                         if constexpr (OFF) {
 #pragma unroll
                             for (int h = 0; h < 2; h++) {
-                                const float z = scale_word(h * QO + Q);
+                                const float z = scale_value(sw[G & 1], Q, h);
                                 acc[h][0] += z * xsum[0];
                                 acc[h][1] += z * xsum[1];
                                 acc[h][2] += z * xsum[2];
@@ -343,12 +370,12 @@ __global__ __launch_bounds__(W * 64) void lut_batch_kernel(MatvecArgs a)
                     }
                 });
             } else {
-            static_for<4>([&](auto G) {   // the four 128-k groups of the k-block
+            static_for<4 * GSUB>([&](auto G) {   // the scale groups of the k-block
                     constexpr int r = G;
                     float4v part[CH];
                     float4v xsum = zero4;
-                    static_for<4>([&](auto TT) {
-                        constexpr int t = 4 * r + TT;   // MFMA t: chunks 4 t .. 4 t + 3
+                    static_for<SG>([&](auto TT) {
+                        constexpr int t = SG * r + TT;   // MFMA t: chunks 4 t .. 4 t + 3
                         const half8 xa = *reinterpret_cast<const __attribute__((address_space(3))) half8 *>(xr + t * 16);
                         static_for<CH>([&](auto I) {
                             const uint32_t word = t < 4 ? R[I].x : t < 8 ? R[I].y : t < 12 ? R[I].z : R[I].w;
@@ -362,7 +389,7 @@ __global__ __launch_bounds__(W * 64) void lut_batch_kernel(MatvecArgs a)
                     });
                     static_for<CH>([&](auto I) {
                         constexpr int U = u0 + I, b = U / 2, h = U % 2;
-                        const float s = scale_of(r, h * QO + b);
+                        const float s = scale_of(r, b, h);
                         acc[h][0] += s * part[I][0];
                         acc[h][1] += s * part[I][1];
                         acc[h][2] += s * part[I][2];
@@ -371,7 +398,7 @@ __global__ __launch_bounds__(W * 64) void lut_batch_kernel(MatvecArgs a)
                     if constexpr (OFF && C == 0 && NU <= 6) {
 #pragma unroll
                         for (int h = 0; h < 2; h++) {
-                            const float z = scale_of(r, h * QO + Q);
+                            const float z = scale_of(r, Q, h);
                             acc[h][0] += z * xsum[0];
                             acc[h][1] += z * xsum[1];
                             acc[h][2] += z * xsum[2];
@@ -384,17 +411,17 @@ __global__ __launch_bounds__(W * 64) void lut_batch_kernel(MatvecArgs a)
             __builtin_amdgcn_sched_barrier(0);   // one pass after the other: keeps the registers of a pass apart
         });
         if constexpr (OFF && NU > 6) {   // many planes: the offset term in a pass of its own
-            static_for<4>([&](auto G) {
+            static_for<4 * GSUB>([&](auto G) {
                 constexpr int r = G;
                 float4v xsum = zero4;
-                static_for<4>([&](auto TT) {
-                    constexpr int t = 4 * r + TT;
+                static_for<SG>([&](auto TT) {
+                    constexpr int t = SG * r + TT;
                     const half8 xa = *reinterpret_cast<const __attribute__((address_space(3))) half8 *>(xr + t * 16);
                     xsum = __builtin_amdgcn_mfma_f32_16x16x32_f16(xa, __builtin_bit_cast(half8, ones), xsum, 0, 0, 0);
                 });
 #pragma unroll
                 for (int h = 0; h < 2; h++) {
-                    const float z = scale_of(r, h * QO + Q);
+                    const float z = scale_of(r, Q, h);
                     acc[h][0] += z * xsum[0];
                     acc[h][1] += z * xsum[1];
                     acc[h][2] += z * xsum[2];
@@ -441,45 +468,63 @@ __global__ __launch_bounds__(W * 64) void lut_batch_kernel(MatvecArgs a)
         for (int v = 0; v < 4; v++) complete_output(arrival[h][v], valid[h][v], word[h][v], yout[h][v], a.k_splits);
 }
 
-template <int Q, bool OFF, int W, bool TWO>
+template <int Q, bool OFF, int GSUB, int W, bool TWO>
 hipError_t launch_batch_w(const MatvecArgs &a, int workgroups, int waves, hipStream_t stream)
 {
+    constexpr int QO = Q + (OFF ? 1 : 0);
     static std::atomic<unsigned long long> allowed{0};
     int dev = 0;
     hipError_t e = hipGetDevice(&dev);
     if (e != hipSuccess) return e;
     const unsigned long long bit = 1ull << (dev & 63);
     if (!(allowed.load(std::memory_order_relaxed) & bit)) {
-        e = hipFuncSetAttribute(reinterpret_cast<const void *>(&lut_batch_kernel<Q, OFF, W, TWO>),
-                                hipFuncAttributeMaxDynamicSharedMemorySize, batch_lds_bytes(W));
+        e = hipFuncSetAttribute(reinterpret_cast<const void *>(&lut_batch_kernel<Q, OFF, GSUB, W, TWO>),
+                                hipFuncAttributeMaxDynamicSharedMemorySize, batch_lds_bytes(batch_waves_max(GSUB, QO), GSUB, QO));
         if (e != hipSuccess) return e;
         allowed.fetch_or(bit, std::memory_order_relaxed);
     }
-    hipLaunchKernelGGL((lut_batch_kernel<Q, OFF, W, TWO>), dim3(workgroups), dim3(waves * kLanes), batch_lds_bytes(waves), stream,
-                       a);
+    hipLaunchKernelGGL((lut_batch_kernel<Q, OFF, GSUB, W, TWO>), dim3(workgroups), dim3(waves * kLanes),
+                       batch_lds_bytes(waves, GSUB, QO), stream, a);
     return hipGetLastError();
 }
 
-template <int Q>
-hipError_t launch_batch_off(int has_offset, const MatvecArgs &a, int wg, int waves, hipStream_t s)
+template <int Q, bool OFF, int GSUB>
+hipError_t launch_batch_two(const MatvecArgs &a, int wg, int waves, hipStream_t s)
 {
     constexpr int W = kBatchWaves;
-    if (waves < kBatchWavesMin || waves > W) return hipErrorInvalidValue;
-    if (a.rows > waves)
-        return has_offset ? launch_batch_w<Q, true, W, true>(a, wg, waves, s) : launch_batch_w<Q, false, W, true>(a, wg, waves, s);
-    return has_offset ? launch_batch_w<Q, true, W, false>(a, wg, waves, s) : launch_batch_w<Q, false, W, false>(a, wg, waves, s);
+    if (waves < kBatchWavesMin || waves > batch_waves_max(GSUB, Q + (OFF ? 1 : 0))) return hipErrorInvalidValue;
+    return a.rows > waves ? launch_batch_w<Q, OFF, GSUB, W, true>(a, wg, waves, s)
+                          : launch_batch_w<Q, OFF, GSUB, W, false>(a, wg, waves, s);
+}
+
+template <int Q>
+hipError_t launch_batch_off(int has_offset, int gsub, const MatvecArgs &a, int wg, int waves, hipStream_t s)
+{
+    if (has_offset) {
+        switch (gsub) {
+            case 1: return launch_batch_two<Q, true, 1>(a, wg, waves, s);
+            case 2: return launch_batch_two<Q, true, 2>(a, wg, waves, s);
+            default: return launch_batch_two<Q, true, 4>(a, wg, waves, s);
+        }
+    }
+    switch (gsub) {
+        case 1: return launch_batch_two<Q, false, 1>(a, wg, waves, s);
+        case 2: return launch_batch_two<Q, false, 2>(a, wg, waves, s);
+        default: return launch_batch_two<Q, false, 4>(a, wg, waves, s);
+    }
 }
 
 }  // namespace
 
-hipError_t launch_batch(int q, int has_offset, const MatvecArgs &a, int workgroups, int waves, hipStream_t stream)
+hipError_t launch_batch(int q, int has_offset, int gsub, const MatvecArgs &a, int workgroups, int waves, hipStream_t stream)
 {
     if (a.rows < 1 || a.rows > kBatchRows) return hipErrorInvalidValue;
+    if (gsub != 1 && gsub != 2 && gsub != 4) return hipErrorInvalidValue;
     switch (q) {
-        case 1: return launch_batch_off<1>(has_offset, a, workgroups, waves, stream);
-        case 2: return launch_batch_off<2>(has_offset, a, workgroups, waves, stream);
-        case 3: return launch_batch_off<3>(has_offset, a, workgroups, waves, stream);
-        case 4: return launch_batch_off<4>(has_offset, a, workgroups, waves, stream);
+        case 1: return launch_batch_off<1>(has_offset, gsub, a, workgroups, waves, stream);
+        case 2: return launch_batch_off<2>(has_offset, gsub, a, workgroups, waves, stream);
+        case 3: return launch_batch_off<3>(has_offset, gsub, a, workgroups, waves, stream);
+        case 4: return launch_batch_off<4>(has_offset, gsub, a, workgroups, waves, stream);
         default: return hipErrorInvalidValue;   // more planes than kBatchMaxPlanes
     }
 }

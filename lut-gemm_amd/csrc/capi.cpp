@@ -208,7 +208,7 @@ double batch_plan_cost(const Shape &s, int cus, int waves, int ks, Plan *out)
 
 Plan choose_batch_plan(const Shape &s, int cus)
 {
-    const int wmax = lutgemm_kernels::kBatchWaves, wmin = lutgemm_kernels::kBatchWavesMin;
+    const int wmax = lutgemm_kernels::batch_waves_max(s.gsub, s.qo), wmin = lutgemm_kernels::kBatchWavesMin;
     Plan best{wmax, div_up(s.nb, wmax), s.ts, 1};
     double best_cost = 1e30;
     long best_wgs = 0;
@@ -232,7 +232,7 @@ Plan choose_batch_plan(const Shape &s, int cus)
 
 bool batch_kernel_takes(const Shape &s)
 {
-    return s.gsub == 1 && s.q <= lutgemm_kernels::kBatchMaxPlanes;
+    return s.q <= lutgemm_kernels::kBatchMaxPlanes;
 }
 
 // A handle's device memory belongs to the device that was current when it was created.
@@ -536,7 +536,7 @@ int run_matvec(const lutgemm_weight *w, const void *x, void *y, int m, void *str
                 a.y_stride = 1;
                 a.y_row_stride = s.n;
             }
-            hipError_t e = lutgemm_kernels::launch_batch(s.q, s.has_offset, a, plan.ntiles * plan.k_splits, plan.waves, st);
+            hipError_t e = lutgemm_kernels::launch_batch(s.q, s.has_offset, s.gsub, a, plan.ntiles * plan.k_splits, plan.waves, st);
             if (e != hipSuccess) {
                 if (static_ws && r > 0) g_static_dirty[w->device] = true;
                 return hip_fail(e, "launch lut_batch_kernel");
@@ -1077,7 +1077,7 @@ int lutgemm_weight_autotune(lutgemm_weight *w, void *stream)
         const int rows = bi ? kRowsPerPass : 8;
         struct Timed { float ms; double cost; Plan p; };
         std::vector<Timed> timed;
-        for (int waves = lutgemm_kernels::kBatchWavesMin; waves <= lutgemm_kernels::kBatchWaves; waves++)
+        for (int waves = lutgemm_kernels::kBatchWavesMin; waves <= lutgemm_kernels::batch_waves_max(s.gsub, s.qo); waves++)
             for (int ks = 1; ks <= s.ts && ks <= kMaxSplits; ks++) {
                 Plan p;
                 const double cost = batch_plan_cost(s, w->compute_units, waves, ks, &p);

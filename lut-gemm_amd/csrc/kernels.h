@@ -56,13 +56,28 @@ hipError_t launch_matvec(int q, int has_offset, int gsub, const MatvecArgs &a, i
 hipError_t launch_matvec_multi(int q, int has_offset, int gsub, const MultiMatvecArgs &m, int workgroups, int waves,
                                hipStream_t stream);
 
-// 1..kBatchRows activation rows in one pass (matrix cores); scale layouts with gsub == 1 and up to
-// kBatchMaxPlanes planes only.  A workgroup has kBatchWavesMin .. kBatchWaves wavefronts:
+// 1..kBatchRows activation rows in one pass (matrix cores); up to kBatchMaxPlanes planes.  A workgroup has kBatchWavesMin .. kBatchWaves wavefronts:
 // wavefront w stages activation rows w and w + wavefronts, so eight cover the 16 rows of a pass.
 constexpr int kBatchMaxPlanes = 4;
 constexpr int kBatchWaves = 16;
 constexpr int kBatchWavesMin = 8;
-hipError_t launch_batch(int q, int has_offset, const MatvecArgs &a, int workgroups, int waves, hipStream_t stream);
+// LDS of a workgroup of the batch kernel: the pattern table (64 KiB), two activation blocks of 17
+// rows of 1040 bytes, and per wavefront a 1 KiB staging area plus the scales of its tile for the
+// matrix lanes (one scale group per 128 k: the lanes' scale words as they are, up to 5; two or four
+// groups per 128 k: 4 bytes per (group, plane or offset, output pair)).  A compute unit has 160 KiB,
+// which bounds the wavefronts of a workgroup when there are four groups per 128 k.
+constexpr int batch_scale_area_bytes(int gsub, int qo) { return gsub == 1 ? 256 * 5 : 256 * gsub * qo; }
+constexpr int batch_lds_bytes(int waves, int gsub, int qo)
+{
+    return 256 * 16 * 16 + 2 * 17 * 1040 + waves * (1024 + batch_scale_area_bytes(gsub, qo));
+}
+constexpr int batch_waves_max(int gsub, int qo)
+{
+    int w = kBatchWaves;
+    while (w > kBatchWavesMin && batch_lds_bytes(w, gsub, qo) > 160 * 1024) w--;
+    return w;
+}
+hipError_t launch_batch(int q, int has_offset, int gsub, const MatvecArgs &a, int workgroups, int waves, hipStream_t stream);
 
 // words[0..count) = 0 (a fill kernel rather than a memset node, so that it can be captured)
 hipError_t launch_fill_zero(unsigned long long *words, size_t count, hipStream_t stream);

@@ -17,11 +17,11 @@ def default_dense_threshold(weight):
     """Rows up to which the packed routes beat dequantised weight + library GEMM (measured on
     MI355X at k = n = 12288 and k = 12288, n = 49152; LutLinear(dense_threshold=...) overrides).
 
-    Shapes the batch kernel takes (group size a multiple of 128, up to four planes): one pass of
-    16 rows costs 21-37 us against 50 us for the GEMM, two passes 40-72 us against 56 us: 32 rows
-    for one or two planes, 16 for three or four.  Other shapes go through two-row passes of the
-    table-lookup kernel, which lose to the GEMM from three rows on."""
-    if weight.group_size % 128 == 0 and weight.nb <= 4:
+    Weights of up to four planes go through the batch kernel: one pass of 16 rows costs 21-49 us
+    (one to four planes, group sizes 128 down to 32) against 50 us for the GEMM, two passes 40-98 us
+    against 56 us: 32 rows for one or two planes, 16 for three or four.  More planes go through
+    two-row passes of the table-lookup kernel, which lose to the GEMM from three rows on."""
+    if weight.nb <= 4:
         return 32 if weight.nb <= 2 else 16
     return 2
 

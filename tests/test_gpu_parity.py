@@ -143,7 +143,7 @@ def test_row_pairs_equal_single_rows_bit_for_bit(lutgemm, oracle, device, k, n, 
     """A two-row pass must give each row exactly as a one-row launch with the same plan produces
     it (same tables, same order of accumulation), for every scale layout (g % 128, % 64, % 32),
     with and without offset, for several plans.  Five rows go two per pass as well when the
-    group size is not a multiple of 128 (then equally bit-identical); otherwise the batch kernel
+    weight has more than four planes (then equally bit-identical); otherwise the batch kernel
     takes them in one pass, within the tolerance."""
     from lutgemm import synth
     m = 5
@@ -160,7 +160,7 @@ def test_row_pairs_equal_single_rows_bit_for_bit(lutgemm, oracle, device, k, n, 
             y1 = run_matvec(lutgemm, W, x[r:r + 1], device)
             if r < 2:
                 assert np.array_equal(y2[r].view(np.uint16), y1[0].view(np.uint16)), "row %d of 2, plan %s" % (r, W.plan())
-            if g % 128 != 0:
+            if q > 4:
                 assert np.array_equal(y[r].view(np.uint16), y1[0].view(np.uint16)), "row %d plan %s" % (r, W.plan())
     W.close()
 
@@ -191,12 +191,17 @@ def test_many_rows(lutgemm, oracle, device, k, n, q, g, offset):
 @pytest.mark.parametrize("k,n,q,g,offset", [
     (1024, 40, 4, 128, True), (2048, 33, 1, 128, False), (1536, 100, 1, 256, True), (640, 70, 2, 128, True),
     (4096, 96, 4, 4096, False), (896, 513, 3, 128, True), (3072, 1000, 3, 384, False), (12288, 320, 4, 128, True),
+    # two and four scale groups per 128 k (group sizes 64 / 192 and 32 / 96)
+    (1024, 40, 4, 64, True), (2048, 33, 1, 32, False), (1536, 100, 2, 96, True), (640, 70, 3, 32, True),
+    (3072, 1000, 3, 64, False), (1152, 513, 2, 192, True), (12288, 320, 4, 32, True), (4096, 96, 1, 64, True),
+    (2048, 200, 2, 32, False), (2048, 200, 2, 64, False),
 ])
 def test_batch_kernel_shapes(lutgemm, oracle, device, k, n, q, g, offset):
-    """Three and more rows with a group size that is a multiple of 128 and up to four planes go
-    through the weight once on the matrix cores: every plane count, with and without offset, k that
-    ends inside a k-block, n that ends inside a batch, one to many k-splits, row counts below, at
-    and above the 16 rows of a pass; deterministic; row- and column-batched forms agree."""
+    """Three and more rows with up to four planes go through the weight once on the matrix cores:
+    every plane count and every scale-group layout (one, two or four groups per 128 k), with and
+    without offset, k that ends inside a k-block, n that ends inside a batch, one to many k-splits,
+    row counts below, at and above the 16 rows of a pass; deterministic; row- and column-batched
+    forms agree."""
     from lutgemm import synth
     w, W = make(lutgemm, synth, k, n, q, g, offset=offset, seed=k + 5 * q)
     ts = (k + 511) // 512

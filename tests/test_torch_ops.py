@@ -98,12 +98,12 @@ def test_operator_argument_checks(lutgemm, device):
 
 
 def test_default_dense_threshold_follows_the_weight(lutgemm, device):
-    """Shapes the batch kernel takes keep the packed route for one or two passes of 16 rows,
-    every other shape leaves it from three rows on."""
+    """Weights the batch kernel takes (up to four planes) keep the packed route for one or two
+    passes of 16 rows, the others leave it from three rows on."""
     from lutgemm import quantize, torch_ops
     print("case default dense threshold", flush=True)
     lin, _ = _layer(5, out_f=64, in_f=512, bias=False)
-    for qbits, g, want in ((2, 128, 32), (4, 128, 16), (3, 64, 2), (5, 128, 2)):
+    for qbits, g, want in ((2, 128, 32), (4, 128, 16), (3, 64, 16), (1, 32, 32), (5, 128, 2)):
         c, _ = quantize.quantize_linear(lin.weight.detach(), qbits, g, "rtn", rounds=0)
         layer = torch_ops.LutLinear(c)
         assert layer.dense_threshold == want, (qbits, g, layer.dense_threshold)
