@@ -145,6 +145,7 @@ class Point:
         self.xd = torch.from_numpy(self.x16).to(dev)
         self.yd = torch.zeros((copies, m, n), dtype=torch.float16, device=dev)
         self.plan = first.plan()
+        self.plan_m = first.plan(m)
 
     def items(self, count, rotate=True, offset=0):
         out = []
@@ -229,7 +230,7 @@ def point_record(pt, us, us_hot):
             "fused_independent_us_per_matvec": pt.fused_us,
             "fused_independent_pct_hbm_peak": pt.b_w / pt.fused_us / 1e3 / HBM_PEAK_GBS * 100,
             "hot_us_per_matvec": us_hot, "packed_weight_bytes": pt.b_w, "weight_copies_rotated": pt.copies,
-            "plan_of_one_row_launches" if pt.m > 1 else "plan": pt.plan}
+            "plan": pt.plan_m, "plan_of_one_row_launches": pt.plan}
 
 
 def base_line(args, metric, value, us, workload, extra_config=None):

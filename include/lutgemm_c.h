@@ -189,6 +189,13 @@ int lutgemm_weight_unpack(const lutgemm_weight *w, uint32_t *bW, uint16_t *alpha
 int lutgemm_weight_plan(const lutgemm_weight *w, int *workgroups, int *waves_per_group,
                         int *k_splits, int *k_blocks_per_group);
 
+/* The same for the launches a call with m activation rows makes (m = 1: the plan above; m = 2:
+ * the two-row plan; m >= 3: the batch kernel's plan for passes of min(m, 16) rows where the
+ * weight has up to four planes, else the two-row plan).  LUTGEMM_ERR_BAD_SHAPE for m outside
+ * 1..LUTGEMM_MAX_BATCH.  No counterpart in the reference. */
+int lutgemm_weight_plan_for(const lutgemm_weight *w, int m, int *workgroups, int *waves_per_group,
+                            int *k_splits, int *k_blocks_per_group);
+
 /* Override the launch plan, for one-row and two-row launches alike (0 keeps the automatic
  * choice for that field); synchronises the device first.  Returns LUTGEMM_ERR_BAD_SHAPE if the request cannot be launched
  * (1..12 waves per workgroup, 1..min(k/512 rounded up, 128) k-splits). */

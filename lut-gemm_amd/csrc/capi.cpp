@@ -917,6 +917,24 @@ int lutgemm_weight_plan(const lutgemm_weight *w, int *workgroups, int *waves_per
     return LUTGEMM_OK;
 }
 
+int lutgemm_weight_plan_for(const lutgemm_weight *w, int m, int *workgroups, int *waves_per_group, int *k_splits,
+                            int *k_blocks_per_group)
+{
+    if (!w) return fail(LUTGEMM_ERR_NULL_POINTER, "null argument to weight_plan_for");
+    if (m < 1 || m > LUTGEMM_MAX_BATCH)
+        return fail(LUTGEMM_ERR_BAD_SHAPE, "m=%d outside 1..%d", m, LUTGEMM_MAX_BATCH);
+    Plan p = m == 1 ? w->plan : w->plan2;
+    if (m >= 3 && batch_kernel_takes(w->shape)) {
+        const int pass_rows = m < kRowsPerPass ? m : kRowsPerPass;
+        p = w->batch_measured[pass_rows > 8] ? w->plan_batch[pass_rows > 8] : choose_batch_plan(w->shape, w->compute_units);
+    }
+    if (workgroups) *workgroups = p.ntiles * p.k_splits;
+    if (waves_per_group) *waves_per_group = p.waves;
+    if (k_splits) *k_splits = p.k_splits;
+    if (k_blocks_per_group) *k_blocks_per_group = p.blocks_per_split;
+    return LUTGEMM_OK;
+}
+
 int lutgemm_weight_set_plan(lutgemm_weight *w, int waves_per_group, int k_splits)
 {
     if (!w) return fail(LUTGEMM_ERR_NULL_POINTER, "null argument to weight_set_plan");

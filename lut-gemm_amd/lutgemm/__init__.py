@@ -27,7 +27,7 @@ MAX_BATCH = 4096
 EXPORTED = [
     "lutgemm_weight_create", "lutgemm_weight_create_f16", "lutgemm_weight_destroy", "lutgemm_weight_info",
     "lutgemm_matvec", "lutgemm_matvec_cols", "lutgemm_matvec_many", "lutgemm_dequantize", "lutgemm_weight_unpack",
-    "lutgemm_weight_plan", "lutgemm_weight_set_plan", "lutgemm_weight_autotune", "lutgemm_weight_device_ptrs", "lutgemm_packed_sizes",
+    "lutgemm_weight_plan", "lutgemm_weight_plan_for", "lutgemm_weight_set_plan", "lutgemm_weight_autotune", "lutgemm_weight_device_ptrs", "lutgemm_packed_sizes",
     "lutgemm_pack_host", "lutgemm_unpack_host", "lutgemm_float_to_half", "lutgemm_last_error",
     "lutgemm_status_string", "lutgemm_version", "lutgemm_pack_file", "lutgemm_unpack_file", "lutgemm_weight_save",
     "lutgemm_weight_load", "lutgemm_weight_clone", "lutgemm_read_probe", "lutgemm_dense_gemv_f16",
@@ -85,6 +85,7 @@ def load():
     L.lutgemm_dequantize.argtypes = [vp, vp, i, vp]
     L.lutgemm_weight_unpack.argtypes = [vp, vp, vp, vp]
     L.lutgemm_weight_plan.argtypes = [vp, pi, pi, pi, pi]
+    L.lutgemm_weight_plan_for.argtypes = [vp, ctypes.c_int, pi, pi, pi, pi]
     L.lutgemm_pack_file.argtypes = [vp, vp, vp, i, i, i, i, ctypes.c_char_p]
     L.lutgemm_unpack_file.argtypes = [ctypes.c_char_p, vp, vp, vp, ctypes.POINTER(WeightInfo)]
     L.lutgemm_weight_save.argtypes = [vp, ctypes.c_char_p]
@@ -246,9 +247,10 @@ class BCQWeight:
         _check(load().lutgemm_weight_info(self._h, ctypes.byref(info)))
         return info
 
-    def plan(self):
+    def plan(self, m=1):
+        """Launch plan of calls with m activation rows (one-row, two-row or batch kernel)."""
         v = [ctypes.c_int() for _ in range(4)]
-        _check(load().lutgemm_weight_plan(self._h, *[ctypes.byref(x) for x in v]))
+        _check(load().lutgemm_weight_plan_for(self._h, m, *[ctypes.byref(x) for x in v]))
         return dict(workgroups=v[0].value, waves=v[1].value, k_splits=v[2].value, k_blocks=v[3].value)
 
     def set_plan(self, waves=0, k_splits=0):

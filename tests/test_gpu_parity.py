@@ -264,7 +264,10 @@ def test_autotune_keeps_results_and_picks_a_valid_plan(lutgemm, oracle, device):
     # the batch kernel (measured plans for passes of up to 8 and of 9..16 rows): another order
     # of additions, same tolerance
     for m in (3, 5, 12):
-        assert_within_tolerance(run_matvec(lutgemm, W, x[:m], device), truth[:m], "m=%d" % m)
+        bp = W.plan(m)
+        assert 8 <= bp["waves"] <= 16 and bp["workgroups"] == -(-(n // 32) // bp["waves"]) * bp["k_splits"], bp
+        assert_within_tolerance(run_matvec(lutgemm, W, x[:m], device), truth[:m], "m=%d plan=%s" % (m, bp))
+    assert W.plan(2)["k_splits"] == plan["k_splits"] and W.plan(1) == plan
     W.close()
 
 
@@ -322,7 +325,8 @@ def test_device_round_trip_and_dequantize(lutgemm, oracle, device):
 def test_random_shapes_plans_and_batches(lutgemm, oracle, device):
     """Sixty seeded random problems: ragged k (any multiple of 32, so the last k-block and the
     last scale group are partial), odd n, every q, group sizes with all three scale layouts,
-    with / without offset, 1..6 rows, random launch plans."""
+    with / without offset, 1..33 rows (one-row, two-row and batch kernels, more than one pass),
+    random launch plans."""
     from lutgemm import synth
     rng = np.random.default_rng(20240607)
     for case in range(60):
@@ -332,7 +336,7 @@ def test_random_shapes_plans_and_batches(lutgemm, oracle, device):
         k = g * G
         n = int(rng.integers(1, 700))
         offset = bool(rng.integers(0, 2))
-        m = int(rng.integers(1, 7))
+        m = int(rng.choice([1, 1, 2, 2, 3, 4, 5, 6, 8, 9, 12, 16, 17, 20, 33]))
         ts = (k + 511) // 512
         waves = int(rng.integers(0, 13))
         ks = int(rng.integers(0, ts + 1))
