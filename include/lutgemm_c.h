@@ -201,6 +201,12 @@ int lutgemm_weight_plan_for(const lutgemm_weight *w, int m, int *workgroups, int
  * (1..12 waves per workgroup, 1..min(k/512 rounded up, 128) k-splits). */
 int lutgemm_weight_set_plan(lutgemm_weight *w, int waves_per_group, int k_splits);
 
+/* Override the batch kernel's launch plan (calls with 3 or more rows on weights of up to four
+ * planes): 8..16 wavefronts per workgroup and the k-splits; both 0: back to the automatic choice.
+ * LUTGEMM_ERR_BAD_SHAPE if the request cannot be launched, LUTGEMM_ERR_UNSUPPORTED for weights
+ * that never take the batch kernel.  No launch on the handle may be in flight. */
+int lutgemm_weight_set_batch_plan(lutgemm_weight *w, int waves_per_group, int k_splits);
+
 /* Measure the most promising launch plans on the device (a few launches each, on `stream`, with
  * scratch activations of its own) and keep the fastest, separately for launches with one
  * activation row and for two-row passes (which keep the k-split of the one-row plan, so that

@@ -935,6 +935,31 @@ int lutgemm_weight_plan_for(const lutgemm_weight *w, int m, int *workgroups, int
     return LUTGEMM_OK;
 }
 
+int lutgemm_weight_set_batch_plan(lutgemm_weight *w, int waves_per_group, int k_splits)
+{
+    if (!w) return fail(LUTGEMM_ERR_NULL_POINTER, "null argument to weight_set_batch_plan");
+    const Shape &s = w->shape;
+    if (!batch_kernel_takes(s))
+        return fail(LUTGEMM_ERR_UNSUPPORTED, "weights of more than %d planes do not go through the batch kernel",
+                    lutgemm_kernels::kBatchMaxPlanes);
+    if (waves_per_group == 0 && k_splits == 0) {   // back to the model's choice
+        w->batch_measured[0] = w->batch_measured[1] = false;
+        return LUTGEMM_OK;
+    }
+    const int wmax = lutgemm_kernels::batch_waves_max(s.gsub, s.qo);
+    if (waves_per_group < lutgemm_kernels::kBatchWavesMin || waves_per_group > wmax)
+        return fail(LUTGEMM_ERR_BAD_SHAPE, "waves_per_group=%d outside %d..%d", waves_per_group,
+                    lutgemm_kernels::kBatchWavesMin, wmax);
+    if (k_splits < 1 || k_splits > s.ts || k_splits > kMaxSplits)
+        return fail(LUTGEMM_ERR_BAD_SHAPE, "k_splits=%d outside 1..%d", k_splits, s.ts < kMaxSplits ? s.ts : kMaxSplits);
+    Plan p;
+    if (batch_plan_cost(s, w->compute_units, waves_per_group, k_splits, &p) < 0.0)
+        return fail(LUTGEMM_ERR_BAD_SHAPE, "k_splits=%d leaves a k-split without k-blocks (%d k-blocks)", k_splits, s.ts);
+    w->plan_batch[0] = w->plan_batch[1] = p;
+    w->batch_measured[0] = w->batch_measured[1] = true;
+    return LUTGEMM_OK;
+}
+
 int lutgemm_weight_set_plan(lutgemm_weight *w, int waves_per_group, int k_splits)
 {
     if (!w) return fail(LUTGEMM_ERR_NULL_POINTER, "null argument to weight_set_plan");

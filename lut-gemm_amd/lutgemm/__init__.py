@@ -27,7 +27,7 @@ MAX_BATCH = 4096
 EXPORTED = [
     "lutgemm_weight_create", "lutgemm_weight_create_f16", "lutgemm_weight_destroy", "lutgemm_weight_info",
     "lutgemm_matvec", "lutgemm_matvec_cols", "lutgemm_matvec_many", "lutgemm_dequantize", "lutgemm_weight_unpack",
-    "lutgemm_weight_plan", "lutgemm_weight_plan_for", "lutgemm_weight_set_plan", "lutgemm_weight_autotune", "lutgemm_weight_device_ptrs", "lutgemm_packed_sizes",
+    "lutgemm_weight_plan", "lutgemm_weight_plan_for", "lutgemm_weight_set_plan", "lutgemm_weight_set_batch_plan", "lutgemm_weight_autotune", "lutgemm_weight_device_ptrs", "lutgemm_packed_sizes",
     "lutgemm_pack_host", "lutgemm_unpack_host", "lutgemm_float_to_half", "lutgemm_last_error",
     "lutgemm_status_string", "lutgemm_version", "lutgemm_pack_file", "lutgemm_unpack_file", "lutgemm_weight_save",
     "lutgemm_weight_load", "lutgemm_weight_clone", "lutgemm_read_probe", "lutgemm_dense_gemv_f16",
@@ -86,6 +86,7 @@ def load():
     L.lutgemm_weight_unpack.argtypes = [vp, vp, vp, vp]
     L.lutgemm_weight_plan.argtypes = [vp, pi, pi, pi, pi]
     L.lutgemm_weight_plan_for.argtypes = [vp, ctypes.c_int, pi, pi, pi, pi]
+    L.lutgemm_weight_set_batch_plan.argtypes = [vp, ctypes.c_int, ctypes.c_int]
     L.lutgemm_pack_file.argtypes = [vp, vp, vp, i, i, i, i, ctypes.c_char_p]
     L.lutgemm_unpack_file.argtypes = [ctypes.c_char_p, vp, vp, vp, ctypes.POINTER(WeightInfo)]
     L.lutgemm_weight_save.argtypes = [vp, ctypes.c_char_p]
@@ -255,6 +256,10 @@ class BCQWeight:
 
     def set_plan(self, waves=0, k_splits=0):
         _check(load().lutgemm_weight_set_plan(self._h, waves, k_splits))
+
+    def set_batch_plan(self, waves=0, k_splits=0):
+        """Launch plan of the batch kernel (3 or more rows); defaults: back to the automatic choice."""
+        _check(load().lutgemm_weight_set_batch_plan(self._h, waves, k_splits))
 
     def autotune(self, stream=0):
         """Measure candidate launch plans on the device and keep the fastest; returns the plan."""

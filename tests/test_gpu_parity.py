@@ -245,6 +245,34 @@ def test_every_launch_plan_agrees(lutgemm, oracle, device):
     W.close()
 
 
+@pytest.mark.parametrize("k,n,q,g,offset", [(4096, 520, 2, 128, True), (2048, 200, 3, 64, False), (6144, 97, 1, 32, True),
+                                            (8192, 1000, 4, 256, False)])
+def test_every_batch_plan_agrees(lutgemm, oracle, device, k, n, q, g, offset):
+    """The batch kernel under forced launch plans: 8..16 wavefronts per workgroup (fewer than, as
+    many as and more than the batch has rows), one to many k-splits.  Every plan meets the
+    tolerance and repeats bit for bit; a request that cannot be launched is refused."""
+    from lutgemm import synth
+    w, W = make(lutgemm, synth, k, n, q, g, offset=offset, seed=k + n)
+    ts = (k + 511) // 512
+    x = synth.make_x(16, k, seed=n)
+    truth = truth_of(oracle, w, x)
+    for waves, ks in ((8, 1), (12, 2), (16, ts // 2), (10, ts), (16, 2), (14, 1), (9, 2)):
+        for m in (8, 5, 3, 12, 16):
+            say("case batch plan", k, n, q, g, offset, waves, ks, m)
+            W.set_batch_plan(waves, ks)
+            bp = W.plan(m)
+            assert bp["waves"] == waves and bp["workgroups"] == -(-(-(-n // 32)) // waves) * bp["k_splits"], (bp, waves, ks)
+            y = run_matvec(lutgemm, W, x[:m], device)
+            assert_within_tolerance(y, truth[:m], "m=%d waves=%d ks=%d plan=%s" % (m, waves, ks, bp))
+            assert np.array_equal(y.view(np.uint16), run_matvec(lutgemm, W, x[:m], device, cols=True).view(np.uint16))
+    for waves, ks in ((7, 1), (17, 1), (8, ts + 1), (8, 0)):
+        with pytest.raises(lutgemm.LutGemmError):
+            W.set_batch_plan(waves, ks)
+    W.set_batch_plan()   # back to the model's choice
+    assert_within_tolerance(run_matvec(lutgemm, W, x[:8], device), truth[:8], "model plan %s" % W.plan(8))
+    W.close()
+
+
 def test_autotune_keeps_results_and_picks_a_valid_plan(lutgemm, oracle, device):
     import torch
     from lutgemm import synth
