@@ -235,6 +235,43 @@ bool batch_kernel_takes(const Shape &s)
     return s.q <= lutgemm_kernels::kBatchMaxPlanes;
 }
 
+// Launch shape of several independent batches in one grid (lutgemm_matvec_many): one number of
+// wavefronts per workgroup and one number of k-blocks per workgroup for all entries, with the
+// per-k-block and per-wavefront times of the batch kernel's model; a workgroup also pays its own
+// start and end (pattern table, first tile, split-k atomics), the launch is paid once.
+FusedPlan choose_fused_batch_plan(const Shape *const *shapes, int count, int cus)
+{
+    const double block_us = 1.82, group_us = 6.0;
+    int max_ts = 1, wmax = lutgemm_kernels::kBatchWaves;
+    for (int e = 0; e < count; e++) {
+        max_ts = shapes[e]->ts > max_ts ? shapes[e]->ts : max_ts;
+        const int w = lutgemm_kernels::batch_waves_max(shapes[e]->gsub, shapes[e]->qo);
+        wmax = w < wmax ? w : wmax;
+    }
+    FusedPlan best{wmax, max_ts};
+    double best_cost = 1e300;
+    for (int waves = lutgemm_kernels::kBatchWavesMin; waves <= wmax; waves++)
+        for (int bpg = div_up(max_ts, kMaxSplits); bpg <= max_ts; bpg++) {
+            long groups = 0;
+            double work = 0.0;  // summed time of all workgroups
+            for (int e = 0; e < count; e++) {
+                const Shape &s = *shapes[e];
+                const int b = bpg < s.ts ? bpg : s.ts;
+                const long g = (long)div_up(s.nb, waves) * div_up(s.ts, b);
+                groups += g;
+                work += (double)g * (b * (waves * 0.0635 * s.q + block_us) + group_us);
+            }
+            const double per_group = work / (double)groups;
+            const long rounds = (groups + cus - 1) / cus;
+            const double cost = (double)rounds * per_group;
+            if (cost < best_cost - 1e-9) {
+                best_cost = cost;
+                best = FusedPlan{waves, bpg};
+            }
+        }
+    return best;
+}
+
 // A handle's device memory belongs to the device that was current when it was created.
 int check_device(const lutgemm_weight *w)
 {
@@ -754,27 +791,36 @@ int lutgemm_matvec_many(const lutgemm_weight *const *ws, const void *const *xs, 
     if (count < 0) return fail(LUTGEMM_ERR_BAD_SHAPE, "count=%d is negative", count);
     struct Range { uintptr_t lo, hi; };
     auto overlap = [](const Range &a, const Range &b) { return a.lo < b.hi && b.lo < a.hi; };
+    // what one launch can take: one-row entries (table-lookup kernel) or batches of 3 to 16 rows of
+    // weights the batch kernel takes; anything else (two rows, more than 16, more than four
+    // planes with several rows) is launched on its own
+    auto kind_of = [](const lutgemm_weight *w, int m) {
+        if (m == 1) return 1;
+        if (m >= 3 && m <= kRowsPerPass && batch_kernel_takes(w->shape)) return 2;
+        return 0;
+    };
     int i = 0;
     while (i < count) {
-        // Longest run of entries starting at i that one launch can take: one activation row each,
-        // the same kernel instance, no handle twice (its split-k words would be shared), and no
-        // output overlapping an input or output of another entry of the run, so that their order
-        // does not matter.  Anything else goes through its own launch, in order.
+        // Longest run of entries starting at i that one launch can take: the same kind and kernel
+        // instance, no handle twice (its split-k words would be shared), and no output overlapping
+        // an input or output of another entry of the run, so that their order does not matter.
+        // Anything else goes through its own launch, in order.
         lutgemm_kernels::MultiMatvecArgs multi{};
         Range xr[lutgemm_kernels::kMaxFused], yr[lutgemm_kernels::kMaxFused];
         const Shape *shapes[lutgemm_kernels::kMaxFused];
         int j = i;
         const lutgemm_weight *w0 = ws[i];
-        for (; j < count && j - i < lutgemm_kernels::kMaxFused; j++) {
+        const int kind = w0 && xs[i] && ys[i] ? kind_of(w0, ms[i]) : 0;
+        for (; kind != 0 && j < count && j - i < lutgemm_kernels::kMaxFused; j++) {
             const lutgemm_weight *w = ws[j];
-            if (!w || !xs[j] || !ys[j] || ms[j] != 1 || ((uintptr_t)xs[j] & 15u) != 0) break;
+            if (!w || !xs[j] || !ys[j] || ((uintptr_t)xs[j] & 15u) != 0 || kind_of(w, ms[j]) != kind) break;
             const Shape &s = w->shape;
             if (s.q != w0->shape.q || s.has_offset != w0->shape.has_offset || s.gsub != w0->shape.gsub ||
                 w->device != w0->device)
                 break;
             const int e = j - i;
-            xr[e] = Range{(uintptr_t)xs[j], (uintptr_t)xs[j] + (size_t)s.k * 2};
-            yr[e] = Range{(uintptr_t)ys[j], (uintptr_t)ys[j] + (size_t)s.n * 2};
+            xr[e] = Range{(uintptr_t)xs[j], (uintptr_t)xs[j] + (size_t)ms[j] * s.k * 2};
+            yr[e] = Range{(uintptr_t)ys[j], (uintptr_t)ys[j] + (size_t)ms[j] * s.n * 2};
             bool independent = true;
             for (int p = 0; p < e && independent; p++)
                 independent = ws[i + p] != w && !overlap(yr[e], yr[p]) && !overlap(yr[e], xr[p]) && !overlap(xr[e], yr[p]);
@@ -790,7 +836,10 @@ int lutgemm_matvec_many(const lutgemm_weight *const *ws, const void *const *xs, 
             a.x = xs[j];
             a.y = ys[j];
             a.y_stride = 1;
-            a.rows = 1;
+            a.rows = ms[j];
+            a.x_row_stride = s.k;
+            a.y_row_stride = s.n;
+            a.accum_row_stride = (long long)s.nb * kBatch;
         }
         const int run = j - i;
         if (run < 2) {
@@ -800,7 +849,8 @@ int lutgemm_matvec_many(const lutgemm_weight *const *ws, const void *const *xs, 
             continue;
         }
         if (int st_dev = check_device(w0)) return st_dev;
-        const FusedPlan fp = choose_fused_plan(shapes, run, w0->compute_units);
+        const FusedPlan fp = kind == 1 ? choose_fused_plan(shapes, run, w0->compute_units)
+                                       : choose_fused_batch_plan(shapes, run, w0->compute_units);
         int blocks = 0;
         for (int e = 0; e < run; e++) {
             lutgemm_kernels::MatvecArgs &a = multi.entry[e];
@@ -813,9 +863,11 @@ int lutgemm_matvec_many(const lutgemm_weight *const *ws, const void *const *xs, 
             if (int st_ws = stream_words(const_cast<lutgemm_weight *>(ws[i + e]), stream, &a.accum, &slot)) return st_ws;
         }
         multi.count = run;
-        hipError_t e = lutgemm_kernels::launch_matvec_multi(w0->shape.q, w0->shape.has_offset, w0->shape.gsub, multi,
-                                                            blocks, fp.waves, static_cast<hipStream_t>(stream));
-        if (e != hipSuccess) return hip_fail(e, "launch lut_matvec_multi_kernel");
+        hipError_t e = kind == 1 ? lutgemm_kernels::launch_matvec_multi(w0->shape.q, w0->shape.has_offset, w0->shape.gsub, multi,
+                                                                       blocks, fp.waves, static_cast<hipStream_t>(stream))
+                                 : lutgemm_kernels::launch_batch_multi(w0->shape.q, w0->shape.has_offset, w0->shape.gsub, multi,
+                                                                       blocks, fp.waves, static_cast<hipStream_t>(stream));
+        if (e != hipSuccess) return hip_fail(e, kind == 1 ? "launch lut_matvec_multi_kernel" : "launch lut_batch_kernel");
         i = j;
     }
     return LUTGEMM_OK;

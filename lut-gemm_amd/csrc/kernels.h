@@ -78,6 +78,11 @@ constexpr int batch_waves_max(int gsub, int qo)
     return w;
 }
 hipError_t launch_batch(int q, int has_offset, int gsub, const MatvecArgs &a, int workgroups, int waves, hipStream_t stream);
+// A work list of independent batches in one launch: entries sharing q, has_offset, gsub and the
+// wavefronts per workgroup, each with 1..kBatchRows rows and its own ntiles / k_splits / blocks_per_split;
+// workgroups = sum of the entries' ntiles * k_splits, entry i starting at first_block[i].
+hipError_t launch_batch_multi(int q, int has_offset, int gsub, const MultiMatvecArgs &m, int workgroups, int waves,
+                              hipStream_t stream);
 
 // words[0..count) = 0 (a fill kernel rather than a memset node, so that it can be captured)
 hipError_t launch_fill_zero(unsigned long long *words, size_t count, hipStream_t stream);

@@ -109,10 +109,16 @@ __device__ __forceinline__ Arrival arrive_output(float total, bool valid, unsign
 }
 
 // Second half: the lane whose add arrived last writes the output and clears the word.
-__device__ __forceinline__ void complete_output(const Arrival &r, bool valid, unsigned long long *word, __half *yout,
-                                                int k_splits)
+// arrived_last only looks at the answer of the atomic; a wavefront that finishes several values per
+// lane evaluates it for all of them before the first finish_last, so that no wait for an answer
+// comes behind a store (the wait would then also wait for that store's round trip).
+__device__ __forceinline__ bool arrived_last(const Arrival &r, bool valid, int k_splits)
 {
-    if (!valid || (r.old >> 56) != (unsigned long long)(k_splits - 1)) return;
+    return valid && (r.old >> 56) == (unsigned long long)(k_splits - 1);
+}
+
+__device__ __forceinline__ void finish_last(const Arrival &r, unsigned long long *word, __half *yout, int k_splits)
+{
     const unsigned long long all = r.old + r.addend;
     const long long value = (long long)(all & (kPosInfFlag - 1)) - (long long)k_splits * (1ll << 46);
     float result = __ll2float_rn(value) * (1.f / 16777216.f);
@@ -121,6 +127,12 @@ __device__ __forceinline__ void complete_output(const Arrival &r, bool valid, un
         result = flags == kPosInfFlag ? __builtin_inff() : flags == kNegInfFlag ? -__builtin_inff() : __builtin_nanf("");
     *yout = __float2half_rn(result);
     __hip_atomic_store(word, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+__device__ __forceinline__ void complete_output(const Arrival &r, bool valid, unsigned long long *word, __half *yout,
+                                                int k_splits)
+{
+    if (arrived_last(r, valid, k_splits)) finish_last(r, word, yout, k_splits);
 }
 
 __device__ __forceinline__ void finish_output(float total, bool active, int out, int lane, __half *y,

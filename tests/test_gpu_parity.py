@@ -484,6 +484,87 @@ def test_matvec_many_shares_launches_and_keeps_every_result(lutgemm, oracle, dev
         W.close()
 
 
+def test_matvec_many_fuses_batches(lutgemm, oracle, device):
+    """Independent batches of 3 to 16 rows share one launch of the batch kernel, whatever their
+    shapes and row counts (more rows than the launch has wavefronts per workgroup included); runs
+    are cut where the kind of entry changes (one row, two rows, more than 16, another plane count),
+    where a handle repeats and where an entry reads an earlier output.  Every entry meets the
+    tolerance against the oracle, the call repeats bit for bit, and entries launched on their own
+    equal their own lutgemm_matvec call bit for bit."""
+    import torch
+    from lutgemm import synth
+    st = torch.cuda.current_stream().cuda_stream
+    shapes = [(2048, 1024, 2, 128, False), (2048, 1000, 2, 128, False), (4096, 2048, 2, 256, False),
+              (1536, 520, 2, 128, False), (2048, 1024, 2, 64, False), (2048, 1024, 3, 128, False)]
+    ws = [make(lutgemm, synth, k, n, q, g, offset=off, seed=70 + i) for i, (k, n, q, g, off) in enumerate(shapes)]
+    clones = [ws[0][1].clone() for _ in range(3)]
+    xh = {k: synth.make_x(20, k, seed=k + 1) for k in (1536, 2048, 4096)}
+    xs = {k: torch.from_numpy(v).to(device) for k, v in xh.items()}
+
+    def buf(n, m):
+        return torch.full((m, n), float("nan"), dtype=torch.float16, device=device)
+
+    entries = []            # (weight, x tensor, y tensor, m, synthetic weight or None, host x, exact?)
+    def add(W, w, k, m, exact, x=None, hx=None):
+        x = xs[k][:m] if x is None else x
+        entries.append((W, x, buf(W.mSize, m), m, w, xh[k][:m] if hx is None and w is not None else hx, exact))
+    add(ws[0][1], ws[0][0], 2048, 8, False)       # a run of batches: equal shapes, other n, other k and g, ragged k
+    add(clones[0], ws[0][0], 2048, 3, False)
+    add(ws[1][1], ws[1][0], 2048, 16, False)      # 16 rows: more than the wavefronts of a workgroup may be
+    add(ws[2][1], ws[2][0], 4096, 5, False)
+    add(ws[3][1], ws[3][0], 1536, 12, False)
+    add(ws[4][1], ws[4][0], 2048, 8, True)        # g = 64: another kernel instance, alone between two runs
+    add(clones[1], ws[0][0], 2048, 4, False)      # a second run ...
+    add(clones[2], ws[0][0], 2048, 9, False)
+    add(ws[0][1], ws[0][0], 2048, 2, True)        # ... cut by two rows (table-lookup kernel)
+    add(ws[1][1], ws[1][0], 2048, 1, False)       # one row entries form a run of their own kind
+    add(ws[3][1], ws[3][0], 1536, 1, False)
+    add(ws[5][1], ws[5][0], 2048, 8, True)        # three planes: alone
+    add(ws[0][1], ws[0][0], 2048, 20, True)       # more than 16 rows: two passes, alone
+    add(ws[0][1], ws[0][0], 2048, 8, False)       # the same handle right after itself: a new run starts here
+    add(clones[0], ws[0][0], 2048, 8, False)
+    # an entry that reads the previous entry's output cannot share its launch
+    wsq, Wsq = make(lutgemm, synth, 1024, 1024, 2, 128, offset=False, seed=99)
+    Wsq2 = Wsq.clone()
+    xsq_h = synth.make_x(8, 1024, seed=5)
+    xsq = torch.from_numpy(xsq_h).to(device)
+    chain_in = buf(1024, 8)
+    entries.append((Wsq, xsq, chain_in, 8, wsq, xsq_h, False))
+    entries.append((Wsq2, chain_in, buf(1024, 8), 8, None, None, False))
+    want = []
+    for W, x, y, m, _, _, _ in entries:
+        ref = torch.full_like(y, float("nan"))
+        W.matvec(x.data_ptr(), ref.data_ptr(), m, st)
+        torch.cuda.synchronize()
+        if y is chain_in:
+            chain_in.copy_(ref)       # the next reference call reads it
+        want.append(ref)
+    seq = lutgemm.MatvecSequence([(e[0], e[1].data_ptr(), e[2].data_ptr(), e[3]) for e in entries])
+    first = None
+    for rep in range(3):
+        for e in entries:
+            e[2].fill_(float("nan"))
+        seq.launch(st)
+        torch.cuda.synchronize()
+        got = [e[2].clone() for e in entries]
+        for idx, (e, ref, y) in enumerate(zip(entries, want, got)):
+            say("case many batches entry", idx, "rep", rep)
+            if e[6]:
+                assert torch.equal(y.view(torch.int16), ref.view(torch.int16)), "entry %d, repetition %d" % (idx, rep)
+            if rep == 0 and e[4] is not None:
+                assert_within_tolerance(y.cpu().numpy(), truth_of(oracle, e[4], e[5]), "entry %d" % idx)
+        # the chained entry saw the finished output of the entry before it
+        assert_within_tolerance(got[-1].cpu().numpy(), truth_of(oracle, wsq, got[-2].cpu().numpy()), "chained entry")
+        if first is None:
+            first = got
+        else:
+            assert all(torch.equal(a.view(torch.int16), b.view(torch.int16)) for a, b in zip(first, got)), rep
+    for c in clones + [Wsq, Wsq2]:
+        c.close()
+    for _, W in ws:
+        W.close()
+
+
 def test_one_handle_on_two_streams(lutgemm, oracle, device):
     """Every stream that launches on a handle has split-k words of its own: launches that
     overlap on two streams give the results of the same launches issued one after the other."""
