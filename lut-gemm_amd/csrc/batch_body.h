@@ -147,8 +147,12 @@ __device__ __forceinline__ void batch_workgroup(const MatvecArgs &a, unsigned bl
     constexpr int SG = 4 / GSUB;    // matrix instructions per scale group (a k-block has 4 GSUB groups)
     constexpr int SUBL = 16 / GSUB; // lanes of a row that share a scale group
     constexpr int NU = 2 * Q;   // sign vectors (units) of a tile: unit U = plane U / 2, output half U % 2
-    constexpr int CH = NU <= 6 ? NU : NU % 6 == 0 ? 6 : NU % 5 == 0 ? 5 : NU % 4 == 0 ? 4 : 2;   // units per pass
-    constexpr int P = Q <= 2 ? LUTGEMM_BATCH_AHEAD : 0;   // steps of LDS reads in flight ahead of the matrix instructions (0: the compiler's order)
+    // Steps of LDS reads in flight ahead of the matrix instructions (0: the compiler's order), and the
+    // sign vectors taken per pass over the k-block.  Up to three planes the reads are placed by hand
+    // (three planes in two passes of three vectors: the registers of six do not fit); four planes
+    // keep the compiler's order (with reads ahead they spill).
+    constexpr int P = Q <= 3 ? LUTGEMM_BATCH_AHEAD : 0;
+    constexpr int CH = P > 0 ? (NU <= 4 ? NU : 3) : NU <= 6 ? NU : NU % 6 == 0 ? 6 : NU % 5 == 0 ? 5 : NU % 4 == 0 ? 4 : 2;
     // The kernel's only LDS object, so it starts at LDS address 0: pattern addresses are formed
     // from the sign byte and a lane constant alone.
     extern __shared__ __attribute__((aligned(16))) unsigned char lds_generic[];
@@ -351,7 +355,7 @@ __device__ __forceinline__ void batch_workgroup(const MatvecArgs &a, unsigned bl
                         after_wait(bits[slot][I]);
                         part[I] = __builtin_amdgcn_mfma_f32_16x16x32_f16(xa[slot], bits[slot][I], TT == 0 ? zero4 : part[I], 0, 0, 0);
                     });
-                    if constexpr (OFF)
+                    if constexpr (OFF && C == 0)   // the offset term once per k-block, with the first pass
                         xsum = __builtin_amdgcn_mfma_f32_16x16x32_f16(xa[slot], __builtin_bit_cast(half8, ones),
                                                                       TT == 0 ? zero4 : xsum, 0, 0, 0);
                     if constexpr (TT == SG - 1) {
@@ -364,7 +368,7 @@ __device__ __forceinline__ void batch_workgroup(const MatvecArgs &a, unsigned bl
                             acc[h][2] += sc * part[I][2];
                             acc[h][3] += sc * part[I][3];
                         });
-                        if constexpr (OFF) {
+                        if constexpr (OFF && C == 0) {
 #pragma unroll
                             for (int h = 0; h < 2; h++) {
                                 const float z = scale_value(sw[G & 1], Q, h);
@@ -417,7 +421,7 @@ __device__ __forceinline__ void batch_workgroup(const MatvecArgs &a, unsigned bl
             }
             __builtin_amdgcn_sched_barrier(0);   // one pass after the other: keeps the registers of a pass apart
         });
-        if constexpr (OFF && NU > 6) {   // many planes: the offset term in a pass of its own
+        if constexpr (OFF && NU > 6 && P == 0) {   // many planes: the offset term in a pass of its own
             static_for<4 * GSUB>([&](auto G) {
                 constexpr int r = G;
                 float4v xsum = zero4;
