@@ -473,17 +473,20 @@ __device__ __forceinline__ void batch_workgroup(const MatvecArgs &a, unsigned bl
     for (int h = 0; h < 2; h++)
 #pragma unroll
         for (int v = 0; v < 4; v++) arrival[h][v] = arrive_output(acc[h][v], valid[h][v], word[h][v]);
-    // every answer is looked at before the first output is written (see arrived_last)
-    bool last[2][4];
+    // Every answer is looked at before the first output is written (see arrived_last): the eight
+    // verdicts go through one register that an empty asm statement pins in front of all stores,
+    // so the compiler cannot sink the wait for a later answer behind an earlier store.
+    unsigned last = 0;
 #pragma unroll
     for (int h = 0; h < 2; h++)
 #pragma unroll
-        for (int v = 0; v < 4; v++) last[h][v] = arrived_last(arrival[h][v], valid[h][v], a.k_splits);
+        for (int v = 0; v < 4; v++) last |= (unsigned)arrived_last(arrival[h][v], valid[h][v], a.k_splits) << (4 * h + v);
+    asm volatile("" : "+v"(last) : : "memory");
 #pragma unroll
     for (int h = 0; h < 2; h++)
 #pragma unroll
         for (int v = 0; v < 4; v++)
-            if (last[h][v]) finish_last(arrival[h][v], word[h][v], yout[h][v], a.k_splits);
+            if (last & (1u << (4 * h + v))) finish_last(arrival[h][v], word[h][v], yout[h][v], a.k_splits);
 }
 
 
