@@ -236,12 +236,18 @@ bool batch_kernel_takes(const Shape &s)
 }
 
 // Launch shape of several independent batches in one grid (lutgemm_matvec_many): one number of
-// wavefronts per workgroup and one number of k-blocks per workgroup for all entries, with the
-// per-k-block and per-wavefront times of the batch kernel's model; a workgroup also pays its own
-// start and end (pattern table, first tile, split-k atomics), the launch is paid once.
-FusedPlan choose_fused_batch_plan(const Shape *const *shapes, int count, int cus)
+// wavefronts per workgroup and one number of k-blocks per workgroup for all entries.  The grid
+// runs in rounds of one workgroup per compute unit.  A workgroup costs a time per tile (more when
+// every wavefront stages two activation rows), a little per k-block, and a start and end of its own
+// that grows with its wavefronts (pattern table, first tiles, the wait for the slowest wavefront);
+// the split-k atomics cost by their number in the whole launch (rows x outputs x k-splits), as
+// the memory side executes them at a fixed rate.  Constants (microseconds) fitted to measured
+// times of 330 plans over eight lists (3 to 12 entries, k and n 2048 to 12288, 1 to 4 planes,
+// 4 to 16 rows) on MI355X; the fit names the fastest measured plan of each list.
+FusedPlan choose_fused_batch_plan(const Shape *const *shapes, const int *rows, int count, int cus)
 {
-    const double block_us = 1.82, group_us = 6.0;
+    const double tile_us = 0.110, two_rows = 1.165, block_us = 0.35, group_us = 3.0, group_wave_us = 0.30;
+    const double atomic_us = 2.5e-6;
     int max_ts = 1, wmax = lutgemm_kernels::kBatchWaves;
     for (int e = 0; e < count; e++) {
         max_ts = shapes[e]->ts > max_ts ? shapes[e]->ts : max_ts;
@@ -253,17 +259,21 @@ FusedPlan choose_fused_batch_plan(const Shape *const *shapes, int count, int cus
     for (int waves = lutgemm_kernels::kBatchWavesMin; waves <= wmax; waves++)
         for (int bpg = div_up(max_ts, kMaxSplits); bpg <= max_ts; bpg++) {
             long groups = 0;
-            double work = 0.0;  // summed time of all workgroups
+            double work = 0.0;     // summed time of all workgroups
+            double atomics = 0.0;  // 64-bit atomics of the launch
             for (int e = 0; e < count; e++) {
                 const Shape &s = *shapes[e];
                 const int b = bpg < s.ts ? bpg : s.ts;
-                const long g = (long)div_up(s.nb, waves) * div_up(s.ts, b);
+                const int ks = div_up(s.ts, b);
+                const long g = (long)div_up(s.nb, waves) * ks;
+                const double tile = tile_us * s.q * (rows[e] > waves ? two_rows : 1.0);
                 groups += g;
-                work += (double)g * (b * (waves * 0.0635 * s.q + block_us) + group_us);
+                work += (double)g * (b * (waves * tile + block_us) + group_us + group_wave_us * waves);
+                if (ks > 1) atomics += (double)s.n * rows[e] * ks;
             }
             const double per_group = work / (double)groups;
             const long rounds = (groups + cus - 1) / cus;
-            const double cost = (double)rounds * per_group;
+            const double cost = (double)rounds * per_group + atomic_us * atomics;
             if (cost < best_cost - 1e-9) {
                 best_cost = cost;
                 best = FusedPlan{waves, bpg};
@@ -808,6 +818,7 @@ int lutgemm_matvec_many(const lutgemm_weight *const *ws, const void *const *xs, 
         lutgemm_kernels::MultiMatvecArgs multi{};
         Range xr[lutgemm_kernels::kMaxFused], yr[lutgemm_kernels::kMaxFused];
         const Shape *shapes[lutgemm_kernels::kMaxFused];
+        int rows_of[lutgemm_kernels::kMaxFused];
         int j = i;
         const lutgemm_weight *w0 = ws[i];
         const int kind = w0 && xs[i] && ys[i] ? kind_of(w0, ms[i]) : 0;
@@ -826,6 +837,7 @@ int lutgemm_matvec_many(const lutgemm_weight *const *ws, const void *const *xs, 
                 independent = ws[i + p] != w && !overlap(yr[e], yr[p]) && !overlap(yr[e], xr[p]) && !overlap(xr[e], yr[p]);
             if (!independent) break;
             shapes[e] = &s;
+            rows_of[e] = ms[j];
             lutgemm_kernels::MatvecArgs &a = multi.entry[e];
             a.signs = w->d_signs;
             a.scales = w->d_scales;
@@ -850,7 +862,7 @@ int lutgemm_matvec_many(const lutgemm_weight *const *ws, const void *const *xs, 
         }
         if (int st_dev = check_device(w0)) return st_dev;
         const FusedPlan fp = kind == 1 ? choose_fused_plan(shapes, run, w0->compute_units)
-                                       : choose_fused_batch_plan(shapes, run, w0->compute_units);
+                                       : choose_fused_batch_plan(shapes, rows_of, run, w0->compute_units);
         int blocks = 0;
         for (int e = 0; e < run; e++) {
             lutgemm_kernels::MatvecArgs &a = multi.entry[e];
