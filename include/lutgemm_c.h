@@ -130,16 +130,16 @@ int lutgemm_matvec_cols(const lutgemm_weight *w, const void *x, void *y, int m, 
 /* `count` matvecs with a single call (a decoder layer's projections, a benchmark loop): entry i
  * computes ys[i] = xs[i] * ws[i] with batch ms[i] exactly as lutgemm_matvec would, and the results
  * are those of the entries executed in order.  Consecutive entries that do not depend on each other
- * share ONE kernel launch (up to 32 per launch): entries that all have one activation row, or that
- * all have 3 to 16 rows on weights of up to four planes (the batch kernel), with the same q /
+ * share ONE kernel launch (up to 32 per launch): entries that all have one activation row, that all
+ * have two, or that all have 3 to 16 rows on weights of up to four planes (the batch kernel), with the same q /
  * offset / group layout, distinct handles, and no output overlapping an input or output of another
  * entry of the launch.  The workgroups of such entries follow each other in one grid, so the memory
  * system stays busy while single workgroups start and finish, and the launch overhead is paid
  * once.  Such a launch has a shape of its own (wavefronts per workgroup, split along k) chosen for
  * the whole run, not the handles' plans, so a result may differ in the last bit from the same
  * entry's lutgemm_matvec call; it is deterministic (same entries, same bits) and within the same
- * tolerance.  Entries that do not qualify (a later entry reading an earlier output, two rows or
- * more than 16, another kernel instance) get launches of their own, in order, exactly as lutgemm_matvec issues them.  Has no counterpart in the reference, whose caller loops over lutGEMM::matmul
+ * tolerance.  Entries that do not qualify (a later entry reading an earlier output, more than 16
+ * rows, three and more rows on more than four planes, another kernel instance) get launches of their own, in order, exactly as lutgemm_matvec issues them.  Has no counterpart in the reference, whose caller loops over lutGEMM::matmul
  * itself (tests/opt/fp16/int3_col_wise_matmul_fp16.cu:120-133).  Stops at the first failing entry. */
 int lutgemm_matvec_many(const lutgemm_weight *const *ws, const void *const *xs, void *const *ys,
                         const int *ms, int count, void *stream);

@@ -146,11 +146,12 @@ Plan choose_plan(const Shape &s, int cus)
 // to measured times of 40 plans over five weight shapes and run lengths 3 to 32 on MI355X.
 struct FusedPlan { int waves, blocks_per_group; };
 
-FusedPlan choose_fused_plan(const Shape *const *shapes, int count, int cus)
+FusedPlan choose_fused_plan(const Shape *const *shapes, int count, int cus, int rows)
 {
-    const double kBytesPerCu = 7.0e6 / 256.0;  // streaming rate per compute unit with all units busy
-    const double kBlockFloor = 1.7;            // a k-block takes at least one loaded memory round trip
-    const double kStartEnd = 2.4, kStartEndPerWave = 0.17;  // per workgroup: 2.4 at 12 wavefronts, more with fewer
+    // two-row passes: a k-block builds and looks up two table sets, bound by the lookups
+    const double kBytesPerCu = (rows == 2 ? 4.8e6 : 7.0e6) / 256.0;  // streaming rate per compute unit with all units busy
+    const double kBlockFloor = rows == 2 ? 2.6 : 1.7;  // a k-block takes at least one loaded memory round trip
+    const double kStartEnd = rows == 2 ? 3.2 : 2.4, kStartEndPerWave = 0.17;  // per workgroup: 2.4 at 12 wavefronts, more with fewer
     const double kPartialExponent = 0.28;      // a round on a fraction f of the units streams f^0.28 as long
     int max_ts = 1;
     for (int e = 0; e < count; e++) max_ts = shapes[e]->ts > max_ts ? shapes[e]->ts : max_ts;
@@ -801,11 +802,12 @@ int lutgemm_matvec_many(const lutgemm_weight *const *ws, const void *const *xs, 
     if (count < 0) return fail(LUTGEMM_ERR_BAD_SHAPE, "count=%d is negative", count);
     struct Range { uintptr_t lo, hi; };
     auto overlap = [](const Range &a, const Range &b) { return a.lo < b.hi && b.lo < a.hi; };
-    // what one launch can take: one-row entries (table-lookup kernel) or batches of 3 to 16 rows of
-    // weights the batch kernel takes; anything else (two rows, more than 16, more than four
-    // planes with several rows) is launched on its own
+    // what one launch can take: one-row entries or two-row entries (table-lookup kernels), or batches
+    // of 3 to 16 rows of weights the batch kernel takes; anything else (more than 16 rows, more than
+    // four planes with three rows and up) is launched on its own
     auto kind_of = [](const lutgemm_weight *w, int m) {
         if (m == 1) return 1;
+        if (m == 2) return 3;
         if (m >= 3 && m <= kRowsPerPass && batch_kernel_takes(w->shape)) return 2;
         return 0;
     };
@@ -861,8 +863,8 @@ int lutgemm_matvec_many(const lutgemm_weight *const *ws, const void *const *xs, 
             continue;
         }
         if (int st_dev = check_device(w0)) return st_dev;
-        const FusedPlan fp = kind == 1 ? choose_fused_plan(shapes, run, w0->compute_units)
-                                       : choose_fused_batch_plan(shapes, rows_of, run, w0->compute_units);
+        const FusedPlan fp = kind == 2 ? choose_fused_batch_plan(shapes, rows_of, run, w0->compute_units)
+                                       : choose_fused_plan(shapes, run, w0->compute_units, kind == 1 ? 1 : 2);
         int blocks = 0;
         for (int e = 0; e < run; e++) {
             lutgemm_kernels::MatvecArgs &a = multi.entry[e];
@@ -875,11 +877,11 @@ int lutgemm_matvec_many(const lutgemm_weight *const *ws, const void *const *xs, 
             if (int st_ws = stream_words(const_cast<lutgemm_weight *>(ws[i + e]), stream, &a.accum, &slot)) return st_ws;
         }
         multi.count = run;
-        hipError_t e = kind == 1 ? lutgemm_kernels::launch_matvec_multi(w0->shape.q, w0->shape.has_offset, w0->shape.gsub, multi,
+        hipError_t e = kind != 2 ? lutgemm_kernels::launch_matvec_multi(w0->shape.q, w0->shape.has_offset, w0->shape.gsub, multi,
                                                                        blocks, fp.waves, static_cast<hipStream_t>(stream))
                                  : lutgemm_kernels::launch_batch_multi(w0->shape.q, w0->shape.has_offset, w0->shape.gsub, multi,
                                                                        blocks, fp.waves, static_cast<hipStream_t>(stream));
-        if (e != hipSuccess) return hip_fail(e, kind == 1 ? "launch lut_matvec_multi_kernel" : "launch lut_batch_kernel");
+        if (e != hipSuccess) return hip_fail(e, kind != 2 ? "launch lut_matvec_multi_kernel" : "launch lut_batch_multi_kernel");
         i = j;
     }
     return LUTGEMM_OK;

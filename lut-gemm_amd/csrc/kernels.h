@@ -52,7 +52,7 @@ struct DequantArgs {
 hipError_t launch_matvec(int q, int has_offset, int gsub, const MatvecArgs &a, int workgroups,
                          int waves, hipStream_t stream);
 
-// entries with rows == 1 sharing q, has_offset, gsub and the wavefronts per workgroup
+// entries that all have one row or all have two, sharing q, has_offset, gsub and the wavefronts per workgroup
 hipError_t launch_matvec_multi(int q, int has_offset, int gsub, const MultiMatvecArgs &m, int workgroups, int waves,
                                hipStream_t stream);
 

@@ -594,7 +594,7 @@ __device__ __forceinline__ void process_tile2(TileRegs<Q, Q + (OFF ? 1 : 0), GSU
 // its tiles.  One 128 KiB table set: it is rebuilt between two barriers at the start of every
 // k-block, while the tile loads of that block (issued one block earlier) are in flight.
 template <int Q, bool OFF, int GSUB>
-__global__ __launch_bounds__(768) void lut_matvec2_kernel(MatvecArgs a)
+__device__ __forceinline__ void matvec2_workgroup(const MatvecArgs &a, int block)
 {
     constexpr int QO = Q + (OFF ? 1 : 0);
     __shared__ float2 table[kTable2Floats / 2];
@@ -603,8 +603,8 @@ __global__ __launch_bounds__(768) void lut_matvec2_kernel(MatvecArgs a)
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int waves = blockDim.x >> 6;
-    const int ntile = blockIdx.x % a.ntiles;
-    const int ks = blockIdx.x / a.ntiles;
+    const int ntile = block % a.ntiles;
+    const int ks = block / a.ntiles;
     const int nb = ntile * waves + wave;
     const bool active = nb < a.nb;
     const int ts0 = ks * a.blocks_per_split;
@@ -683,6 +683,21 @@ __global__ __launch_bounds__(768) void lut_matvec2_kernel(MatvecArgs a)
     asm volatile("" : "+v"(last) : : "memory");
     if (last & 1u) finish_last(r0, w0, y0, a.k_splits);
     if (last & 2u) finish_last(r1, w1, y1, a.k_splits);
+}
+
+template <int Q, bool OFF, int GSUB>
+__global__ __launch_bounds__(768) void lut_matvec2_kernel(MatvecArgs a)
+{
+    matvec2_workgroup<Q, OFF, GSUB>(a, blockIdx.x);
+}
+
+// Several independent two-row passes in one launch, laid out like the one-row work list.
+template <int Q, bool OFF, int GSUB>
+__global__ __launch_bounds__(768) void lut_matvec2_multi_kernel(MultiMatvecArgs m)
+{
+    int i = 0;
+    while (i + 1 < m.count && (int)blockIdx.x >= m.first_block[i + 1]) i++;   // scalar: at most 31 steps
+    matvec2_workgroup<Q, OFF, GSUB>(m.entry[i], (int)blockIdx.x - m.first_block[i]);
 }
 
 // The matvec without its arithmetic: same grid, same tile registers, the same loads in the same
@@ -782,6 +797,10 @@ hipError_t launch_one(const MatvecArgs &a, int workgroups, int threads, hipStrea
 template <int Q, bool OFF, int GSUB>
 hipError_t launch_multi_one(const MultiMatvecArgs &m, int workgroups, int threads, hipStream_t stream)
 {
+    if (m.entry[0].rows > 1) {  // two-row passes (static LDS)
+        hipLaunchKernelGGL((lut_matvec2_multi_kernel<Q, OFF, GSUB>), dim3(workgroups), dim3(threads), 0, stream, m);
+        return hipGetLastError();
+    }
     static std::atomic<unsigned long long> allowed{0};
     const hipError_t e = allow_two_table_sets(&lut_matvec_multi_kernel<Q, OFF, GSUB>, allowed);
     if (e != hipSuccess) return e;

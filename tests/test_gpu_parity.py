@@ -565,6 +565,57 @@ def test_matvec_many_fuses_batches(lutgemm, oracle, device):
         W.close()
 
 
+def test_matvec_many_fuses_two_row_entries(lutgemm, oracle, device):
+    """Independent entries of two rows share one launch of the two-row table-lookup kernel (any
+    number of planes; runs are cut where planes, offset or the scale layout change and where a
+    handle repeats).  Every entry meets the tolerance against the oracle and the call repeats bit
+    for bit; an entry that ends up alone equals its own lutgemm_matvec call bit for bit."""
+    import torch
+    from lutgemm import synth
+    st = torch.cuda.current_stream().cuda_stream
+    shapes = [(2048, 1024, 3, 128, False), (4096, 1000, 3, 128, False), (1536, 520, 3, 256, False),
+              (2048, 1024, 6, 128, False), (2048, 2048, 6, 128, False),
+              (2048, 1024, 3, 128, True), (2048, 1024, 3, 64, False)]
+    ws = [make(lutgemm, synth, k, n, q, g, offset=off, seed=170 + i) for i, (k, n, q, g, off) in enumerate(shapes)]
+    clone = ws[0][1].clone()
+    xh = {k: synth.make_x(2, k, seed=k + 7) for k in (1536, 2048, 4096)}
+    xs = {k: torch.from_numpy(v).to(device) for k, v in xh.items()}
+    order = [0, 1, 2, 3, 4, 5, 6, 0]            # runs: three planes (3), six planes (2), offset alone, g = 64 alone, a single entry
+    entries = []
+    for idx in order:
+        w, W = ws[idx]
+        entries.append((W, xs[w["k"]], torch.full((2, W.mSize), float("nan"), dtype=torch.float16, device=device), w))
+    entries.insert(3, (clone, xs[2048], torch.full((2, clone.mSize), float("nan"), dtype=torch.float16, device=device), ws[0][0]))
+    alone = {len(entries) - 3, len(entries) - 2, len(entries) - 1}
+    want = []
+    for W, x, y, _ in entries:
+        ref = torch.full_like(y, float("nan"))
+        W.matvec(x.data_ptr(), ref.data_ptr(), 2, st)
+        torch.cuda.synchronize()
+        want.append(ref)
+    seq = lutgemm.MatvecSequence([(W, x.data_ptr(), y.data_ptr(), 2) for W, x, y, _ in entries])
+    first = None
+    for rep in range(3):
+        for e in entries:
+            e[2].fill_(float("nan"))
+        seq.launch(st)
+        torch.cuda.synchronize()
+        got = [e[2].clone() for e in entries]
+        for idx, (e, ref, y) in enumerate(zip(entries, want, got)):
+            say("case many two-row entries, entry", idx, "rep", rep)
+            if idx in alone:
+                assert torch.equal(y.view(torch.int16), ref.view(torch.int16)), "entry %d, repetition %d" % (idx, rep)
+            if rep == 0:
+                assert_within_tolerance(y.cpu().numpy(), truth_of(oracle, e[3], xh[e[3]["k"]]), "entry %d" % idx)
+        if first is None:
+            first = got
+        else:
+            assert all(torch.equal(a.view(torch.int16), b.view(torch.int16)) for a, b in zip(first, got)), rep
+    clone.close()
+    for _, W in ws:
+        W.close()
+
+
 def test_one_handle_on_two_streams(lutgemm, oracle, device):
     """Every stream that launches on a handle has split-k words of its own: launches that
     overlap on two streams give the results of the same launches issued one after the other."""
