@@ -5,30 +5,45 @@
 // the whole weight to fp16 in a scratch buffer and calls a library GEMM
 // (lutGEMM/src/kernels.cu:73-79, lutGEMM/src/nQWeight_fp16.cu:93-99).  Here the packed tiles are
 // streamed once, exactly as the one-row kernel streams them, and the batch is contracted on the
-// matrix cores while the tile is in registers:
+// matrix cores while the tile is in registers, without ever writing the signs out as numbers:
 //
-//  * A sign byte (8 consecutive k of one output, one plane) is the B operand of one lane of a
-//    v_mfma_f32_16x16x32_f16: its 8 sign bits become 8 fp16 values +1 / -1 by a 16-byte read from
-//    a constant table in LDS (256 patterns, replicated per lane slot so that the reads are
-//    bank-conflict free).  MFMA lane (kappa = lane / 16, j = lane % 16) supplies output j and, in
-//    MFMA t of a k-block, chunk 4 t + kappa: the four k groups of an MFMA are four neighbouring
-//    chunks, so an MFMA never mixes two scale groups and four MFMAs cover one 128-k group.
-//  * The tiles arrive "k across lanes" (lane = chunk, 16 bytes = 16 outputs).  Per 16-byte sign
-//    vector the wavefront writes its 64 x 16 bytes into a 1 KiB staging area of its own in LDS and
-//    reads them back with two transposing reads (ds_read_b64_tr_b8, a gfx950 instruction: 16 lanes
-//    exchange the bytes of their 8-byte rows inside the LDS unit): lane (kappa, j) then holds the
-//    sign bytes of output j for chunks kappa, kappa + 4, ..., kappa + 60 in MFMA order.  No vector
-//    instruction takes part in the transposition.
-//  * The A operand is the activation block: lane (kappa, i) holds x[row i][8 k of chunk
-//    4 t + kappa], read from an LDS copy that the workgroup shares (rows beyond the batch are zero).
-//  * After the four MFMAs of a group, the 16 x 16 result (rows x outputs) is multiplied by the
-//    fp16 scale of that (plane, group, output) and added to the fp32 accumulators; the offset
-//    term uses the group sums of x, which one more MFMA chain with an all-ones operand provides.
-//    Products of fp16 numbers are exact in fp32, so the only roundings are fp32 additions.
+//  * The contraction is v_smfmac_f32_16x16x64_f16, the matrix instruction for an A operand with
+//    2:4 structured sparsity: of every four consecutive K positions of A two are non-zero, and a
+//    2-bit index per non-zero says which.  The B operand holds every activation twice, as the
+//    pair (-x, +x); the A operand is the constant 1.0; and the SIGN BIT IS THE INDEX: non-zero e
+//    of a lane picks -x or +x of its k.  A sign byte never becomes fp16 numbers, neither through a
+//    table in LDS nor through vector instructions: for the 32 sign bits of a register,
+//        (w & 0x55555555) | 0x88888888      and      ((w >> 1) & 0x55555555) | 0x88888888
+//    are the index registers of four matrix instructions (even k and odd k of four chunks; the
+//    second index of every pair of non-zeros has its high bit set because it addresses positions
+//    2 and 3).  Products 1.0 * (+-x) are exact and the sums are fp32, so the only roundings are
+//    fp32 additions, as in the one-row kernel.
+//  * Operand layout of the instruction (measured on gfx950 with random operands): A lane
+//    (kappa = lane / 16, output = lane % 16) holds non-zeros e = 0..7 for dense positions
+//    K = 16 kappa + 4 (e / 2) + index; the low or high 16 bits of the index register are chosen
+//    by an immediate.  B lane (kb = lane / 16, row = lane % 16) holds K = 8 kb .. 8 kb + 7 in its
+//    first eight halves and K = 32 + 8 kb .. 32 + 8 kb + 7 in the second eight.  C lane
+//    (kappa, row): outputs 4 kappa + v, v = 0..3.
+//  * The tiles arrive "k across lanes" (lane = chunk of 8 k, 16 bytes = 16 outputs).  Per 16-byte
+//    sign vector the wavefront writes its 64 x 16 bytes into a 1 KiB staging area of its own in LDS
+//    and reads them back with two transposing reads (ds_read_b64_tr_b8, a gfx950 instruction: 16
+//    lanes exchange the bytes of their 8-byte rows inside the LDS unit): lane (kappa, output) then
+//    holds the sign bytes of its output for chunks kappa, kappa + 4, ..., kappa + 60; byte b of
+//    word w is chunk kappa + 16 w + 4 b.  Step (w, hh, p) of a k-block takes bytes 2 hh and
+//    2 hh + 1 of word w and the k of parity p: lane kappa contributes k = 8 c + 2 i + p for
+//    c = kappa + 16 w + 8 hh (non-zeros i = 0..3) and c + 4 (non-zeros 4 + i).
+//  * The activation block of a k-block lives in LDS in exactly the form the B operand wants: per
+//    row and (chunk c, parity p) one 16-byte block [-x, +x] x 4 for k = 8 c + p, + 2, + 4, + 6.  A B
+//    lane (kb, row) reads the blocks of chunks base + kb / 2 + 4 (kb % 2) and that + 2.
+//  * After the steps of a scale group, the 16 x 16 result (outputs x rows) is multiplied by the
+//    fp16 scales of that (plane, group) and added to the fp32 accumulators; the offset term uses
+//    the group sums of x, which the same instruction provides with an index that always picks +x.
 //  * At the end every (row, output) goes through the same split-k completion as the one-row kernel.
 //
-// Scale groups of 128 k and more are applied once per four MFMAs; groups of 64 or 32 k (two or
-// four per 128 k) after two or after every MFMA, with the scales re-ordered through LDS first.
+// Scale groups of 128 k and more are applied once per four steps, groups of 64 k after two.  With
+// groups of 32 k a step spans two groups (its chunks c and c + 4); there the scales themselves are
+// the A operand (four times the scale of the first group, four times that of the second) and
+// nothing is multiplied afterwards.
 //
 // This header holds the workgroup body; batch.hip wraps it into the kernel of a single batch,
 // batch_multi.hip into the work-list kernel of lutgemm_matvec_many (two translation units, so that
@@ -47,39 +62,89 @@
 #include "layout.h"
 #include "tile_device.h"
 
-#ifndef LUTGEMM_BATCH_AHEAD
-#define LUTGEMM_BATCH_AHEAD 1
-#endif
-
 namespace lutgemm_kernels {
 using namespace lutgemm_layout;
 
 namespace {
 
 typedef _Float16 half8 __attribute__((ext_vector_type(8)));
+typedef _Float16 half16 __attribute__((ext_vector_type(16)));
 typedef float float4v __attribute__((ext_vector_type(4)));
 typedef __attribute__((address_space(3))) unsigned char lds_byte;
+typedef uint32_t u32x4v __attribute__((ext_vector_type(4)));
 
-constexpr int kPatternBytes = 256 * 16 * 16;               // 64 KiB: [pattern][lane slot][16 bytes]
-constexpr int kXRowBytes = kBlockK * 2 + 16;               // one activation row of a k-block, padded:
-                                                           // 16 rows read at one column hit 64 different banks
-constexpr int kXBufBytes = (kBatchRows + 1) * kXRowBytes;  // 17,680: 16 rows and a spare one that is never read
-static_assert(batch_lds_bytes(0, 1, 1) == kPatternBytes + 2 * kXBufBytes, "kernels.h states the LDS of this kernel");
+// LDS reads whose order and wait counts are fixed by hand.  The compiler waits for every LDS read
+// right before its first use and schedules that use early, which leaves one read in flight per
+// wavefront; the contraction below instead issues the reads of a whole step (the two halves of
+// the B operand, the scales of a group with its last step) ahead of the step before and waits
+// with the count of younger reads (LDS reads of a wavefront return in order; a count that leaves
+// out other younger LDS operations only waits longer).  The asm statements are volatile, so they
+// keep their order among themselves; a result is tied to the wait that covers it by passing
+// through that wait's (or a following empty) asm statement.
+template <int OFFSET>
+__device__ __forceinline__ half8 lds_read128_at(uint32_t addr)
+{
+    half8 v;
+    asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(v) : "v"(addr), "n"(OFFSET));
+    return v;
+}
+template <int OFFSET>
+__device__ __forceinline__ u32x4v lds_read128u_at(uint32_t addr)
+{
+    u32x4v v;
+    asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(v) : "v"(addr), "n"(OFFSET));
+    return v;
+}
+template <int YOUNGER>
+__device__ __forceinline__ void lds_wait(half8 &v)
+{
+    static_assert(YOUNGER >= 0 && YOUNGER <= 15, "lgkmcnt has four bits");
+    asm volatile("s_waitcnt lgkmcnt(%1)" : "+v"(v) : "n"(YOUNGER));
+}
+__device__ __forceinline__ void after_wait(half8 &v) { asm volatile("" : "+v"(v)); }
+__device__ __forceinline__ void after_wait(u32x4v &v) { asm volatile("" : "+v"(v)); }
+__device__ __forceinline__ void after_wait(uint32_t &v) { asm volatile("" : "+v"(v)); }
+template <int OFFSET>
+__device__ __forceinline__ uint32_t lds_read32_at(uint32_t addr)
+{
+    uint32_t v;
+    asm volatile("ds_read_b32 %0, %1 offset:%2" : "=v"(v) : "v"(addr), "n"(OFFSET));
+    return v;
+}
+
+// acc + fp16 half (low or high) of pair * x; written so that the compiler can fold the conversion
+// into a mixed-precision multiply-add (an inline asm instruction here would read the result of a
+// matrix instruction without the wait states the compiler inserts for its own instructions)
+template <bool HIGH>
+__device__ __forceinline__ float fma_half(float acc, uint32_t pair, float x)
+{
+    typedef _Float16 half2v __attribute__((ext_vector_type(2)));
+    const half2v h = __builtin_bit_cast(half2v, pair);
+    return __builtin_fmaf((float)(HIGH ? h.y : h.x), x, acc);
+}
+
+#ifndef LUTGEMM_BATCH_AHEAD
+#define LUTGEMM_BATCH_AHEAD 1
+#endif
+
+// One activation row of a k-block in LDS: 64 chunks x 2 parities x 16 bytes, block (c, p) at
+// 16 * (16 (c % 8) + 2 (c / 8) + p), and 16 bytes of padding: the B lanes of one read differ in
+// row and in c % 8 only, so the 16 lanes the LDS serves together fall into 16 different 16-byte
+// slots modulo 256.
+constexpr int kXRowBytes = kBlockK * 4 + 16;               // 2064
+constexpr int kXBufBytes = (kBatchRows + 1) * kXRowBytes;  // 16 rows and a spare one that is never read
+static_assert(batch_lds_bytes(0, 1, 1) == 2 * kXBufBytes, "kernels.h states the LDS of this kernel");
 constexpr int kStageBytes = 1024;                          // per wavefront: [16 outputs][64 chunk positions]
-// The activation block of k-block ts is 16 rows x 64 chunks of 16 bytes.  Wavefront w moves rows w
-// and w + waves (a launch has at least 8 wavefronts, so two rows per wavefront cover the 16 of a
-// pass), lane = chunk.  The load and the LDS write are separate so that the load of the next block
-// is in flight while the current one is processed.  k beyond the weight and rows beyond the batch
-// read as zero.  No branches: a
-// branch in the loop body costs the register allocator dearly, and with straight-line code the
-// wait counts of the loads stay exact.
+// The activation block of k-block ts is 16 rows x 64 chunks.  Wavefront w moves rows w and
+// w + waves (a launch has at least 8 wavefronts, so two rows per wavefront cover the 16 of a
+// pass); lane L moves chunk 8 (L % 8) + L / 8.  The load and the LDS write are separate so that
+// the load of the next block is in flight while the current one is processed.  k beyond the
+// weight and rows beyond the batch read as zero.  No branches: a branch in the loop body costs
+// the register allocator dearly.
 __device__ __forceinline__ u32x4 load_activation_row(const MatvecArgs &a, int ts, int row, int lane, bool valid)
 {
     const __half *x = reinterpret_cast<const __half *>(a.x);
-    // A row is kept in LDS ordered [kappa = chunk % 4][t = chunk / 4]: position L holds chunk
-    // 4 (L % 16) + L / 16, so that the 16-byte reads of the matrix lanes (kappa, j) at step t fall
-    // into bank groups that depend on j and t only (see the read in the kernel).
-    const int kpos = ts * kBlockK + (4 * (lane & 15) + (lane >> 4)) * kChunk;
+    const int kpos = ts * kBlockK + (8 * (lane & 7) + (lane >> 3)) * kChunk;
     const uint32_t m = 0u - (uint32_t)(valid && row < a.rows && kpos < a.k);
     const size_t offset = ((size_t)row * (size_t)a.x_row_stride + (size_t)kpos) & (size_t)(0 - (long long)(m & 1u));
     u32x4 v = *reinterpret_cast<const u32x4 *>(x + offset);
@@ -90,75 +155,43 @@ __device__ __forceinline__ u32x4 load_activation_row(const MatvecArgs &a, int ts
     return v;
 }
 
+// word (x[2i], x[2i+1]) -> (-x[2i], +x[2i]) (selector 0x01000100) or (-x[2i+1], +x[2i+1]) (0x03020302)
+__device__ __forceinline__ uint32_t minus_plus(uint32_t pair, uint32_t selector)
+{
+    return __builtin_amdgcn_perm(pair, pair, selector) ^ 0x00008000u;
+}
+
 __device__ __forceinline__ void store_activation_row(const u32x4 &v, lds_byte *buf, int row, int lane)
 {
     // rows 16 and up (second rows of the wavefronts of a large workgroup) do not exist: their zeros
     // go to a spare row behind the 16, so that the store needs no branch
     const int slot = row < kBatchRows ? row : kBatchRows;
-    *reinterpret_cast<__attribute__((address_space(3))) u32x4 *>(buf + slot * kXRowBytes + lane * 16) = v;
+    // Chunk c = 8 (lane % 8) + lane / 8: block (c, p) at 16 (16 (c % 8) + 2 (c / 8) + p).  The first
+    // store writes parity (lane / 16) % 2, the second the other one: the 16 lanes the LDS serves
+    // together then differ in (c / 8, parity), that is in their 16-byte slot modulo 256.
+    const int first = (lane >> 4) & 1;
+    lds_byte *at = buf + slot * kXRowBytes + ((lane >> 3) * 16 + (lane & 7) * 2) * 16;
+    const uint32_t sel_a = first ? 0x03020302u : 0x01000100u, sel_b = first ? 0x01000100u : 0x03020302u;
+    *reinterpret_cast<__attribute__((address_space(3))) u32x4 *>(at + 16 * first) =
+        u32x4{minus_plus(v.x, sel_a), minus_plus(v.y, sel_a), minus_plus(v.z, sel_a), minus_plus(v.w, sel_a)};
+    *reinterpret_cast<__attribute__((address_space(3))) u32x4 *>(at + 16 * (first ^ 1)) =
+        u32x4{minus_plus(v.x, sel_b), minus_plus(v.y, sel_b), minus_plus(v.z, sel_b), minus_plus(v.w, sel_b)};
 }
 
-// LDS reads whose order and wait counts are fixed by hand.  The compiler waits for every LDS read
-// right before its first use and schedules that use early, which leaves one read in flight per
-// wavefront; the contraction below instead issues the reads of a whole step (one activation
-// operand, one expanded sign operand per unit) one or two steps ahead and waits with the exact
-// count of younger reads (LDS reads of a wavefront return in order).  The asm statements are
-// volatile, so they keep their order among themselves; a result is tied to the wait that covers
-// it by passing through that wait's (or a following empty) asm statement.
-__device__ __forceinline__ half8 lds_read128(uint32_t addr)
-{
-    half8 v;
-    asm volatile("ds_read_b128 %0, %1" : "=v"(v) : "v"(addr));
-    return v;
-}
-template <int OFFSET>
-__device__ __forceinline__ half8 lds_read128_at(uint32_t addr)
-{
-    half8 v;
-    asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(v) : "v"(addr), "n"(OFFSET));
-    return v;
-}
-template <int OFFSET>
-__device__ __forceinline__ uint32_t lds_read32_at(uint32_t addr)
-{
-    uint32_t v;
-    asm volatile("ds_read_b32 %0, %1 offset:%2" : "=v"(v) : "v"(addr), "n"(OFFSET));
-    return v;
-}
-template <int YOUNGER>
-__device__ __forceinline__ void lds_wait(half8 &v)
-{
-    static_assert(YOUNGER >= 0 && YOUNGER <= 15, "lgkmcnt has four bits");
-    asm volatile("s_waitcnt lgkmcnt(%1)" : "+v"(v) : "n"(YOUNGER));
-}
-__device__ __forceinline__ void after_wait(half8 &v) { asm volatile("" : "+v"(v)); }
-__device__ __forceinline__ void after_wait(uint32_t &v) { asm volatile("" : "+v"(v)); }
-
-// W is the largest number of wavefronts a workgroup may have (it sets the register budget); the
-// launch picks a number from eight up to it that divides the column batches of the shape well
-// over the compute units.  TWO: the batch has more rows than the workgroup has wavefronts, so
-// every wavefront stages a second activation row (a build of its own: the second row's load and
-// store cost the batches that do not need them 2.5 %).
+// TWO: every wavefront stages a second activation row (batches of more rows than the workgroup
+// has wavefronts).
 template <int Q, bool OFF, int GSUB, int W, bool TWO>
 __device__ __forceinline__ void batch_workgroup(const MatvecArgs &a, unsigned block)
 {
     constexpr int QO = Q + (OFF ? 1 : 0);
-    constexpr int SW = GSUB * QO;   // scale words a lane holds per tile
-    constexpr int SG = 4 / GSUB;    // matrix instructions per scale group (a k-block has 4 GSUB groups)
-    constexpr int SUBL = 16 / GSUB; // lanes of a row that share a scale group
-    constexpr int NU = 2 * Q;   // sign vectors (units) of a tile: unit U = plane U / 2, output half U % 2
-    // Steps of LDS reads in flight ahead of the matrix instructions (0: the compiler's order), and the
-    // sign vectors taken per pass over the k-block.  Up to three planes the reads are placed by hand
-    // (three planes in two passes of three vectors: the registers of six do not fit); four planes
-    // keep the compiler's order (with reads ahead they spill).
-    constexpr int P = Q <= 3 ? LUTGEMM_BATCH_AHEAD : 0;
-    constexpr int CH = P > 0 ? (NU <= 4 ? NU : 3) : NU <= 6 ? NU : NU % 6 == 0 ? 6 : NU % 5 == 0 ? 5 : NU % 4 == 0 ? 4 : 2;
-    // The kernel's only LDS object, so it starts at LDS address 0: pattern addresses are formed
-    // from the sign byte and a lane constant alone.
+    constexpr int NU = 2 * Q;            // sign vectors of a tile: plane b, output half h -> 2 b + h
+    constexpr int SW = GSUB * QO;        // scale words of a lane per tile
+    constexpr int SUBL = 16 / GSUB;      // lanes of a tile row per scale sub-row (scale tiles)
+    // the sign vectors taken per pass over the k-block (the registers of more do not fit)
+    constexpr int CH = NU <= 4 ? NU : NU % 3 == 0 ? 3 : 2;
     extern __shared__ __attribute__((aligned(16))) unsigned char lds_generic[];
     lds_byte *lds = (lds_byte *)lds_generic;
-    lds_byte *pattern = lds;
-    lds_byte *xbuf = lds + kPatternBytes;
+    lds_byte *xbuf = lds;
 
     const int tid = threadIdx.x;
     const int threads = blockDim.x;
@@ -171,7 +204,7 @@ __device__ __forceinline__ void batch_workgroup(const MatvecArgs &a, unsigned bl
     const bool active = nb < a.nb;
     const int ts0 = ks * a.blocks_per_split;
     const int ts1 = min(ts0 + a.blocks_per_split, a.ts);
-    lds_byte *stage = lds + kPatternBytes + 2 * kXBufBytes + wave * (kStageBytes + batch_scale_area_bytes(GSUB, QO));
+    lds_byte *stage = lds + 2 * kXBufBytes + wave * (kStageBytes + batch_scale_area_bytes(GSUB, QO));
     lds_byte *scale_area = stage + kStageBytes;
 
     const u32x4 *signs = reinterpret_cast<const u32x4 *>(a.signs);
@@ -179,9 +212,7 @@ __device__ __forceinline__ void batch_workgroup(const MatvecArgs &a, unsigned bl
     const size_t tile0 = (size_t)(active ? nb : 0) * a.ts;
 
     // One tile in registers as in the one-row kernel: the sign vectors and this lane's own scale
-    // words, both fetched one k-block ahead.  The MFMA lanes need the scales of all four 128-k
-    // groups of the k-block for their two outputs (j and 16 + j); group r is held by lane 16 r + j,
-    // so every wavefront passes its scale words through a small LDS area of its own, [word][lane].
+    // words, both fetched one k-block ahead.
     u32x4 sign[NU];
     uint32_t scale[SW];
     {
@@ -192,36 +223,23 @@ __device__ __forceinline__ void batch_workgroup(const MatvecArgs &a, unsigned bl
         for (int u = 0; u < NU; u++) sign[u] = __builtin_nontemporal_load(n0.sign + u * n0.sign_stride);
     }
     __builtin_amdgcn_sched_barrier(0);
-    // Sign patterns: entry e, dword v holds the fp16 pair for bits 2v and 2v+1 of e: +1.0 where
-    // the bit is set, -1.0 where it is clear.  All 16 lane slots of an entry hold the same 16 bytes.
-    for (int idx = tid; idx < 256 * 16; idx += threads) {
-        const uint32_t e = (uint32_t)idx >> 4;
-        u32x4 m;
-        m.x = (((e >> 0) & 1u) ? 0x3c00u : 0xbc00u) | (((e >> 1) & 1u) ? 0x3c000000u : 0xbc000000u);
-        m.y = (((e >> 2) & 1u) ? 0x3c00u : 0xbc00u) | (((e >> 3) & 1u) ? 0x3c000000u : 0xbc000000u);
-        m.z = (((e >> 4) & 1u) ? 0x3c00u : 0xbc00u) | (((e >> 5) & 1u) ? 0x3c000000u : 0xbc000000u);
-        m.w = (((e >> 6) & 1u) ? 0x3c00u : 0xbc00u) | (((e >> 7) & 1u) ? 0x3c000000u : 0xbc000000u);
-        *reinterpret_cast<__attribute__((address_space(3))) u32x4 *>(pattern + idx * 16) = m;
-    }
-    // both activation buffers start at zero
-    for (int idx = tid; idx < 2 * kXBufBytes / 16; idx += threads)
-        *reinterpret_cast<__attribute__((address_space(3))) u32x4 *>(xbuf + idx * 16) = u32x4{0u, 0u, 0u, 0u};
+    // Rows that no wavefront stages (beyond the batch, when the workgroup has fewer wavefronts than
+    // 16) keep whatever the LDS holds: a row is a column of the B operand, and its garbage stays in
+    // the result column of that row, which is never stored.
     u32x4 xrow = load_activation_row(a, ts0, wave, lane, true);
     u32x4 xrow2 = u32x4{0u, 0u, 0u, 0u};
     if constexpr (TWO) xrow2 = load_activation_row(a, ts0, wave + waves, lane, true);
-    __syncthreads();   // the zeros are in place before the first rows go on top of them
     store_activation_row(xrow, xbuf, wave, lane);
     if constexpr (TWO) store_activation_row(xrow2, xbuf, wave + waves, lane);
 
-
-    // lane roles
-    const int kappa = lane >> 4, j = lane & 15;       // MFMA: k group and output column / activation row
+    // lane roles in the matrix instruction
+    const int kappa = lane >> 4, j = lane & 15;
     // Staging.  ds_read_b64_tr_b8 works on rows of 16 lanes: every lane passes the address of an
     // 8-byte row, and lane 8 h + b of the 16 receives byte b of the rows addressed by lanes h, h + 2,
     // ..., h + 14, in that order (measured on gfx950 with tagged bytes).  Lane (kappa, s) addresses
     // outputs 8 (s % 2) .. 8 (s % 2) + 7 of chunk kappa + 4 (s / 2); lane (kappa, j) then receives
     // the sign bytes of output j for chunks kappa + 4 t, t = 0..7, and the same read 512 bytes
-    // further on delivers t = 8..15: together the 16 bytes the contraction consumes.
+    // further on delivers t = 8..15.
     // Lane c (chunk c: kap = c % 4, t = c / 4) writes its 16 bytes to the 16-byte slot
     //     16 (2 (t / 8) + kap / 2) + ((2 (t % 8) + kap % 2) xor 8 (kap / 2)),
     // chosen so that both directions are free of bank conflicts: the 16 lanes the LDS serves together
@@ -237,41 +255,61 @@ __device__ __forceinline__ void batch_workgroup(const MatvecArgs &a, unsigned bl
         reinterpret_cast<__attribute__((address_space(3))) v2i *>(stage + 16 * r_slot + 8 * (j & 1));
     __attribute__((address_space(3))) v2i *stage_r1 =
         reinterpret_cast<__attribute__((address_space(3))) v2i *>(stage + 16 * r_slot + 8 * (j & 1) + 512);
-    // bytes 0, 2 and 3 of a pattern address: lane slot and the LDS address bits above 64 KiB
-    const uint32_t pattern_lane = ((uint32_t)j << 4) + (uint32_t)(size_t)pattern;
 
-    // One group per 128 k: the scale words go to LDS as they are, [word][lane]; the matrix lane
-    // (kappa, j) finds the pair (output j, output 16 + j) of 128-k group r at lane 16 r + j.
+    // Scales.  The matrix lane (kappa, row) needs the scales of its outputs 4 kappa .. 4 kappa + 3 (both
+    // output halves) for every (group of the k-block, plane or offset); the wavefront passes its scale
+    // words through an LDS area of its own so that one 16-byte read delivers them.
+    // One group per 128 k: lane (r = lane / 16, jj = lane % 16) holds, as number hb = h QO + b of its
+    // words, the scale of (group r, plane or offset b, output 16 h + jj).  The words go to LDS as they
+    // are, [word][lane]; the four words d of lanes 16 G + 4 kappa .. + 3 are the numbers 2 d and 2 d + 1
+    // of the lane's four outputs in group G.
     // Two or four groups per 128 k: lane (row r, sub-row sub, jj) holds, in slot t, the scales of
-    // output t SUBL + jj for the group (r, sub); each fp16 number goes to
-    // [group r GSUB + sub][plane or offset][output % 16][output / 16], so that the matrix lanes
-    // again read one word per (group, plane) with the pair (output j, output 16 + j).
+    // output t SUBL + jj for the group r GSUB + sub; every fp16 number goes (2-byte writes) to
+    // [group][plane or offset][(output % 16) / 4][output half][output % 4].
+    // (the halves are read back as wider words: the write type may alias them)
+    typedef uint16_t __attribute__((may_alias)) aliasing_u16;
+    const int s_jj = (lane & 15) % SUBL;
     __attribute__((address_space(3))) uint32_t *scale_w =
         reinterpret_cast<__attribute__((address_space(3))) uint32_t *>(scale_area) + lane;
-    // (the halves are read back as 32-bit words: the write type may alias them)
-    typedef uint16_t __attribute__((may_alias)) aliasing_u16;
     __attribute__((address_space(3))) aliasing_u16 *scale_wh = reinterpret_cast<__attribute__((address_space(3))) aliasing_u16 *>(
-        scale_area + ((((lane >> 4) * GSUB + (lane & 15) / SUBL) * QO) * 16 + (lane & 15) % SUBL) * 4);
-    const __attribute__((address_space(3))) uint32_t *scale_r =
-        reinterpret_cast<const __attribute__((address_space(3))) uint32_t *>(scale_area) + j;
-    // LDS byte offset (from scale_r) of the word of scale group G (0 .. 4 GSUB - 1 of the k-block) that
-    // holds fp16 number hb = half * QO + plane-or-offset (GSUB 1) or the pair of plane-or-offset b
-    auto scale_word_offset = [](int G, int idx) constexpr {
-        return GSUB == 1 ? (idx * kLanes + 16 * G) * 4 : ((G * QO + idx) * 16) * 4;
+        scale_area + (((lane >> 4) * GSUB + (lane & 15) / SUBL) * QO * 32 + (s_jj >> 2) * 8 + (s_jj & 3)) * 2);
+    // (four groups per 128 k: lane (r, sub, jj) holds group 4 r + sub = pair 2 r + sub / 2, half sub % 2)
+    __attribute__((address_space(3))) aliasing_u16 *scale_w4 = reinterpret_cast<__attribute__((address_space(3))) aliasing_u16 *>(
+        scale_area + ((((lane >> 4) * 2 + ((lane >> 3) & 1)) * QO * 32 + (lane & 3)) * 2 + ((lane >> 2) & 1)) * 2);
+    const uint32_t saddr = (uint32_t)(size_t)(scale_area + 16 * kappa);
+    // LDS byte offset (from saddr) of read number rd (0 .. QO - 1) of group G
+    auto scale_read_offset = [](int G, int rd) constexpr { return GSUB == 1 ? rd * 256 + 64 * G : (G * QO + rd) * 64; };
+    // acc + scale of (plane or offset B, output half H, output 4 kappa + V) out of the reads of a group * x
+    auto scale_fma = [](float acc, const u32x4v (&reads)[QO], auto Bc, auto Hc, auto Vc, float x) {
+        constexpr int B = Bc, H = Hc, V = Vc;
+        if constexpr (GSUB == 1) {
+            constexpr int hb = H * QO + B;
+            const u32x4v &w = reads[hb >> 1];
+            return fma_half<(hb & 1) != 0>(acc, V == 0 ? w.x : V == 1 ? w.y : V == 2 ? w.z : w.w, x);
+        } else {
+            const u32x4v &w = reads[B];
+            return fma_half<(V & 1) != 0>(acc, H == 0 ? (V < 2 ? w.x : w.y) : (V < 2 ? w.z : w.w), x);
+        }
     };
-    // the fp16 number of (plane or offset b, output half h) out of the words of one group
-    auto scale_value = [](const uint32_t (&words)[QO], int b, int h) {
-        const int hb = h * QO + b;
-        const uint32_t w = GSUB == 1 ? words[hb >> 1] : words[b];
-        const __half2 h2 = *reinterpret_cast<const __half2 *>(&w);
-        return (GSUB == 1 ? (hb & 1) : h) ? __high2float(h2) : __low2float(h2);
-    };
+
+    // B operand: blocks of chunks base + kb / 2 + 4 (kb % 2) (first eight halves) and that + 2
+    // (512 bytes further on), base = 16 w + 8 hh: block (base + c8, p) sits at 256 c8 + 16 (4 w + 2 hh + p)
+    const int xlane = j * kXRowBytes + ((kappa >> 1) + 4 * (kappa & 1)) * 256;
 
     float4v acc[2];
     acc[0] = float4v{0.f, 0.f, 0.f, 0.f};
     acc[1] = float4v{0.f, 0.f, 0.f, 0.f};
+    // four scale groups per 128 k: an accumulator per output half and unit of a pass, and one per
+    // half for the offset term (see the contraction)
+    float4v acc2[2][2], acc_off[2];
+    acc2[0][0] = acc2[0][1] = acc2[1][0] = acc2[1][1] = acc_off[0] = acc_off[1] = float4v{0.f, 0.f, 0.f, 0.f};
     const float4v zero4 = float4v{0.f, 0.f, 0.f, 0.f};
-    const u32x4 ones = {0x3c003c00u, 0x3c003c00u, 0x3c003c00u, 0x3c003c00u};
+    const half8 ones = {1, 1, 1, 1, 1, 1, 1, 1};
+    constexpr int kAlwaysPlus = (int)0xddddddddu;   // index 1 for the first, 3 for the second non-zero of a pair
+    // (kept in registers, so that the mask and the OR are one v_and_or_b32, which takes no literals)
+    uint32_t mask55 = 0x55555555u, high88 = 0x88888888u;
+    asm("" : "+s"(mask55));
+    asm("" : "+v"(high88));
 
     __syncthreads();
     for (int ts = ts0; ts < ts1; ts++) {
@@ -281,33 +319,32 @@ __device__ __forceinline__ void batch_workgroup(const MatvecArgs &a, unsigned bl
         xrow = load_activation_row(a, ts + 1, wave, lane, more);
         if constexpr (TWO) xrow2 = load_activation_row(a, ts + 1, wave + waves, lane, more);
 
-        // this k-block's scale words into the wavefront's LDS area, then the refill of their registers
+        // this k-block's scales into the wavefront's LDS area, then the refill of their registers
         if constexpr (GSUB == 1) {
 #pragma unroll
             for (int d = 0; d < SW; d++) scale_w[d * kLanes] = scale[d];
-        } else {
+        } else if constexpr (GSUB == 2) {
             static_for<2 * SW>([&](auto F) {
                 constexpr int f = F, t = f / QO, bo = f % QO;   // slot t: output t SUBL + jj
-                constexpr int dest = (bo * 16 + (t % GSUB) * SUBL) * 2 + t / GSUB;   // in fp16 units from scale_wh
-                scale_wh[dest] = (uint16_t)(scale[f >> 1] >> (16 * (f & 1)));
+                constexpr int h = t / GSUB, within = (t % GSUB) * SUBL;
+                scale_wh[bo * 32 + (within / 4) * 8 + h * 4] = (uint16_t)(scale[f >> 1] >> (16 * (f & 1)));
+            });
+        } else {
+            // four groups per 128 k: the scales of the groups 2 P and 2 P + 1 of (plane or offset, output)
+            // side by side in one word, [pair P][plane or offset][output half][output % 16]
+            static_for<2 * SW>([&](auto F) {
+                constexpr int f = F, t = f / QO, bo = f % QO;   // slot t: output 4 t + jj
+                constexpr int h = t / 4;
+                scale_w4[((bo * 2 + h) * 16 + (t % 4) * 4) * 2] = (uint16_t)(scale[f >> 1] >> (16 * (f & 1)));
             });
         }
-        // the reads of these words further down are asm statements or reads through another pointer
-        // type: keep the compiler from moving them above the writes (no instruction is emitted)
+        // the reads of these numbers further down are asm statements: keep the compiler from moving
+        // them above the writes (no instruction is emitted)
         asm volatile("" ::: "memory");
 #pragma unroll
         for (int d = 0; d < SW; d++) scale[d] = __builtin_nontemporal_load(next.scale + d);
-        // the words of scale group G, read when needed (the paths without hand-placed reads)
-        auto scale_of = [&](int G, int b, int h) {
-            const int hb = h * QO + b;
-            const uint32_t w = scale_r[scale_word_offset(G, GSUB == 1 ? hb >> 1 : b) / 4];
-            const __half2 h2 = *reinterpret_cast<const __half2 *>(&w);
-            return (GSUB == 1 ? (hb & 1) : h) ? __high2float(h2) : __low2float(h2);
-        };
 
-        const lds_byte *xr = xbuf + cur * kXBufBytes + j * kXRowBytes + kappa * 256;
-        // The sign vectors are taken CH at a time (all of them up to three planes), so that the
-        // registers of a pass stay within the budget for any number of planes.
+        const lds_byte *xr = xbuf + cur * kXBufBytes + xlane;
         static_for<NU / CH>([&](auto C) {
             constexpr int u0 = C * CH;
             // transpose through the staging area (LDS operations of a wavefront execute in order, so
@@ -322,131 +359,162 @@ __device__ __forceinline__ void batch_workgroup(const MatvecArgs &a, unsigned bl
                 R[I] = u32x4{(uint32_t)lo.x, (uint32_t)lo.y, (uint32_t)hi.x, (uint32_t)hi.y};
                 sign[U] = __builtin_nontemporal_load(next.sign + U * next.sign_stride);
             });
-            if constexpr (P > 0) {
-                // Steps g = 0..15 of the k-block (MFMA t = g: scale group g / SG): the LDS reads of step
-                // g + P are issued before step g is waited for and contracted.
-                half8 xa[P + 1];
-                half8 bits[P + 1][CH];
-                uint32_t sw[2][QO];   // scale words of a group, read with the last step of the group
-                float4v part[CH];
-                float4v xsum = zero4;
-                const uint32_t xaddr = (uint32_t)(size_t)xr, saddr = (uint32_t)(size_t)scale_r;
+            // Steps g = 4 w + 2 hh + p of the k-block.  The LDS reads of step g + P are issued before
+            // step g is waited for and contracted.
+            constexpr int P = LUTGEMM_BATCH_AHEAD;
+            constexpr bool WITH_OFFSET4 = OFF && C == 0;
+            const uint32_t xaddr = (uint32_t)(size_t)xr;
+            if constexpr (GSUB == 4) {
+                // Four scale groups per 128 k: a step covers 64 k of every output, two groups (the lane's
+                // chunks c and c + 4), so the scales go into the A operand instead of 1.0: four times
+                // the scale of the first group, four times that of the second.  The instruction then adds
+                // scale * (+-x) products (exact in fp32) of both groups into one accumulator, for every
+                // plane and group alike, and nothing is left to multiply afterwards.  (With one or two
+                // groups per 128 k this form measured slower than 1.0 and a multiply-add per group: matrix
+                // instructions run slower the more their operand bits vary.)
+                constexpr int NA = CH + (WITH_OFFSET4 ? 2 : 0);   // A operands of a step pair: the units, the offset per half
+                half8 xb0[P + 1], xb1[P + 1], av[NA];
+                uint32_t aw[2][NA];
+                const uint32_t waddr = (uint32_t)(size_t)(scale_area + 4 * j);
                 auto issue = [&](auto Gc) {
-                    constexpr int g = Gc, slot = g % (P + 1);
-                    xa[slot] = lds_read128_at<g * 16>(xaddr);
-                    static_for<CH>([&](auto I) {
-                        const uint32_t word = g < 4 ? R[I].x : g < 8 ? R[I].y : g < 12 ? R[I].z : R[I].w;
-                        constexpr uint32_t sel = 0x03020400u + ((uint32_t)(g & 3) << 8);   // address byte 1 <- sign byte g % 4
-                        bits[slot][I] = lds_read128(__builtin_amdgcn_perm(word, pattern_lane, sel));
-                    });
-                    if constexpr (g % SG == SG - 1)
-                        static_for<QO>([&](auto Wd) { sw[(g / SG) & 1][Wd] = lds_read32_at<scale_word_offset(g / SG, Wd)>(saddr); });
+                    constexpr int g = Gc, slot = g % (P + 1), pair = g / 2;
+                    xb0[slot] = lds_read128_at<16 * g>(xaddr);
+                    xb1[slot] = lds_read128_at<16 * g + 512>(xaddr);
+                    if constexpr (g % 2 == 0)
+                        static_for<NA>([&](auto A) {
+                            constexpr int U = u0 + A, bo = A < CH ? U / 2 : Q, h = A < CH ? U % 2 : A - CH;
+                            aw[pair & 1][A] = lds_read32_at<((pair * QO + bo) * 2 + h) * 64>(waddr);
+                        });
                 };
                 static_for<P>(issue);
                 static_for<16>([&](auto Gc) {
-                    constexpr int g = Gc, G = g / SG, TT = g % SG, slot = g % (P + 1);
+                    constexpr int g = Gc, w = g / 4, hh = (g / 2) % 2, p = g % 2, slot = g % (P + 1), pair = g / 2;
                     if constexpr (g + P < 16) issue(std::integral_constant<int, (g + P < 16 ? g + P : 0)>{});
-                    // reads younger than those of step g: the steps g + 1 .. g + P that exist
-                    constexpr int last = g + P < 16 ? g + P : 15;
-                    // (the scale words of a group are read with its last step: (x + 1) / SG groups end by step x)
-                    constexpr int younger = (last - g) * (1 + CH) + QO * ((last + 1) / SG - (g + 1) / SG);
-                    lds_wait<younger>(xa[slot]);
-                    static_for<CH>([&](auto I) {
-                        after_wait(bits[slot][I]);
-                        part[I] = __builtin_amdgcn_mfma_f32_16x16x32_f16(xa[slot], bits[slot][I], TT == 0 ? zero4 : part[I], 0, 0, 0);
-                    });
-                    if constexpr (OFF && C == 0)   // the offset term once per k-block, with the first pass
-                        xsum = __builtin_amdgcn_mfma_f32_16x16x32_f16(xa[slot], __builtin_bit_cast(half8, ones),
-                                                                      TT == 0 ? zero4 : xsum, 0, 0, 0);
-                    if constexpr (TT == SG - 1) {
-                        static_for<QO>([&](auto Wd) { after_wait(sw[G & 1][Wd]); });
-                        static_for<CH>([&](auto I) {
-                            constexpr int U = u0 + I, b = U / 2, h = U % 2;
-                            const float sc = scale_value(sw[G & 1], b, h);
-                            acc[h][0] += sc * part[I][0];
-                            acc[h][1] += sc * part[I][1];
-                            acc[h][2] += sc * part[I][2];
-                            acc[h][3] += sc * part[I][3];
+                    constexpr int ahead = g + P < 16 ? g + P : 15;
+                    constexpr int younger = 2 * (ahead - g) + NA * ((ahead + 2) / 2 - (g + 2) / 2);
+                    lds_wait<(younger < 15 ? younger : 15)>(xb0[slot]);
+                    after_wait(xb1[slot]);
+                    if constexpr (p == 0)
+                        static_for<NA>([&](auto A) {
+                            after_wait(aw[pair & 1][A]);
+                            const uint32_t word = aw[pair & 1][A];
+                            const uint32_t lo = __builtin_amdgcn_perm(word, word, 0x01000100u), hi = __builtin_amdgcn_perm(word, word, 0x03020302u);
+                            av[A] = __builtin_bit_cast(half8, u32x4v{lo, lo, hi, hi});
                         });
-                        if constexpr (OFF && C == 0) {
-#pragma unroll
-                            for (int h = 0; h < 2; h++) {
-                                const float z = scale_value(sw[G & 1], Q, h);
-                                acc[h][0] += z * xsum[0];
-                                acc[h][1] += z * xsum[1];
-                                acc[h][2] += z * xsum[2];
-                                acc[h][3] += z * xsum[3];
-                            }
-                        }
+                    const half16 xb = __builtin_shufflevector(xb0[slot], xb1[slot], 0, 1, 2, 3, 4, 5, 6, 7, 8, 9, 10, 11, 12, 13, 14, 15);
+                    static_for<CH>([&](auto I) {
+                        constexpr int U = u0 + I, h = U % 2, nth = I / 2;   // the nth unit of this pass with this output half
+                        const uint32_t word = w == 0 ? R[I].x : w == 1 ? R[I].y : w == 2 ? R[I].z : R[I].w;
+                        const int index = (int)(((p ? word >> 1 : word) & mask55) | high88);
+                        acc2[h][nth] = __builtin_amdgcn_smfmac_f32_16x16x64_f16(av[I], xb, acc2[h][nth], index, 0, hh);
+                    });
+                    if constexpr (WITH_OFFSET4) {   // the offset term once per k-block, with the first pass
+                        acc_off[0] = __builtin_amdgcn_smfmac_f32_16x16x64_f16(av[NA - 2], xb, acc_off[0], kAlwaysPlus, 0, 0);
+                        acc_off[1] = __builtin_amdgcn_smfmac_f32_16x16x64_f16(av[NA - 1], xb, acc_off[1], kAlwaysPlus, 0, 0);
                     }
                 });
             } else {
-            static_for<4 * GSUB>([&](auto G) {   // the scale groups of the k-block
-                    constexpr int r = G;
-                    float4v part[CH];
-                    float4v xsum = zero4;
-                    static_for<SG>([&](auto TT) {
-                        constexpr int t = SG * r + TT;   // MFMA t: chunks 4 t .. 4 t + 3
-                        const half8 xa = *reinterpret_cast<const __attribute__((address_space(3))) half8 *>(xr + t * 16);
-                        static_for<CH>([&](auto I) {
-                            const uint32_t word = t < 4 ? R[I].x : t < 8 ? R[I].y : t < 12 ? R[I].z : R[I].w;
-                            constexpr uint32_t sel = 0x03020400u + ((uint32_t)(t & 3) << 8);   // address byte 1 <- sign byte t % 4
-                            const uint32_t addr = __builtin_amdgcn_perm(word, pattern_lane, sel);
-                            const half8 bits = *reinterpret_cast<const __attribute__((address_space(3))) half8 *>(addr);
-                            part[I] = __builtin_amdgcn_mfma_f32_16x16x32_f16(xa, bits, TT == 0 ? zero4 : part[I], 0, 0, 0);
-                        });
-                        if constexpr (OFF && C == 0 && NU <= 6)
-                            xsum = __builtin_amdgcn_mfma_f32_16x16x32_f16(xa, __builtin_bit_cast(half8, ones), xsum, 0, 0, 0);
+            // Steps per scale group: 4 (one group per 128 k) or 2 (two groups).
+            constexpr int STEPS = GSUB == 1 ? 4 : 2;
+            // which of the QO scale reads of a group this pass uses: those of its planes and, with the
+            // first pass, of the offset
+            constexpr bool WITH_OFFSET = OFF && C == 0;
+            auto needed = [](int rd) constexpr {
+                for (int i = 0; i < CH + 2; i++) {
+                    const bool offset_term = i >= CH;
+                    if (offset_term && !WITH_OFFSET) continue;
+                    const int b = offset_term ? Q : (u0 + i) / 2, h = offset_term ? i - CH : (u0 + i) % 2;
+                    if ((GSUB == 1 ? (h * QO + b) >> 1 : b) == rd) return true;
+                }
+                return false;
+            };
+            constexpr int SR = [&]() constexpr { int c = 0; for (int rd = 0; rd < QO; rd++) c += needed(rd) ? 1 : 0; return c; }();   // scale reads with the last step of a group
+            half8 xb0[P + 1], xb1[P + 1];
+            u32x4v sw[2][QO];
+            float4v part[CH];
+            float4v xsum = zero4;
+            auto issue = [&](auto Gc) {
+                constexpr int g = Gc, slot = g % (P + 1), w = g / 4, hh = (g / 2) % 2;
+                constexpr int G = GSUB == 1 ? w : 2 * w + hh;
+                xb0[slot] = lds_read128_at<16 * g>(xaddr);
+                xb1[slot] = lds_read128_at<16 * g + 512>(xaddr);
+                if constexpr (g % STEPS == STEPS - 1)
+                    static_for<QO>([&](auto Bo) {
+                        if constexpr (needed(Bo)) sw[(g / STEPS) & 1][Bo] = lds_read128u_at<scale_read_offset(G, Bo)>(saddr);
+                    });
+            };
+            static_for<P>(issue);
+            static_for<16>([&](auto Gc) {
+                constexpr int g = Gc, w = g / 4, hh = (g / 2) % 2, p = g % 2, slot = g % (P + 1);
+                constexpr bool first = g % STEPS == 0, last = g % STEPS == STEPS - 1;
+                if constexpr (g + P < 16) issue(std::integral_constant<int, (g + P < 16 ? g + P : 0)>{});
+                // reads younger than those of step g: the steps g + 1 .. g + P that exist, two each, and
+                // the scales of the groups that end with one of them
+                constexpr int ahead = g + P < 16 ? g + P : 15;
+                constexpr int younger = 2 * (ahead - g) + SR * ((ahead + 1) / STEPS - (g + 1) / STEPS);
+                lds_wait<(younger < 15 ? younger : 15)>(xb0[slot]);
+                after_wait(xb1[slot]);
+                const half16 xb = __builtin_shufflevector(xb0[slot], xb1[slot], 0, 1, 2, 3, 4, 5, 6, 7, 8, 9, 10, 11, 12, 13, 14, 15);
+                static_for<CH>([&](auto I) {
+                    const uint32_t word = w == 0 ? R[I].x : w == 1 ? R[I].y : w == 2 ? R[I].z : R[I].w;
+                    const int index = (int)(((p ? word >> 1 : word) & mask55) | high88);
+                    part[I] = __builtin_amdgcn_smfmac_f32_16x16x64_f16(ones, xb, first ? zero4 : part[I], index, 0, hh);
+                });
+                if constexpr (WITH_OFFSET)   // the offset term once per k-block, with the first pass
+                    xsum = __builtin_amdgcn_smfmac_f32_16x16x64_f16(ones, xb, first ? zero4 : xsum, kAlwaysPlus, 0, 0);
+                if constexpr (last) {
+                    // (the scale reads were issued with this step's operand reads and are older than
+                    // everything the wait above left in flight)
+                    constexpr int S = (g / STEPS) & 1;
+                    static_for<QO>([&](auto Bo) {
+                        if constexpr (needed(Bo)) after_wait(sw[S][Bo]);
                     });
                     static_for<CH>([&](auto I) {
                         constexpr int U = u0 + I, b = U / 2, h = U % 2;
-                        const float s = scale_of(r, b, h);
-                        acc[h][0] += s * part[I][0];
-                        acc[h][1] += s * part[I][1];
-                        acc[h][2] += s * part[I][2];
-                        acc[h][3] += s * part[I][3];
+                        static_for<4>([&](auto Vc) {
+                            constexpr int v = Vc;
+                            acc[h][v] = scale_fma(acc[h][v], sw[S], std::integral_constant<int, b>{}, std::integral_constant<int, h>{}, Vc, part[I][v]);
+                        });
                     });
-                    if constexpr (OFF && C == 0 && NU <= 6) {
-#pragma unroll
-                        for (int h = 0; h < 2; h++) {
-                            const float z = scale_of(r, Q, h);
-                            acc[h][0] += z * xsum[0];
-                            acc[h][1] += z * xsum[1];
-                            acc[h][2] += z * xsum[2];
-                            acc[h][3] += z * xsum[3];
-                        }
+                    if constexpr (WITH_OFFSET) {
+                        static_for<2>([&](auto Hc) {
+                            static_for<4>([&](auto Vc) {
+                                constexpr int h = Hc, v = Vc;
+                                acc[h][v] = scale_fma(acc[h][v], sw[S], std::integral_constant<int, Q>{}, Hc, Vc, xsum[v]);
+                            });
+                        });
                     }
-                    if constexpr (NU > 6) __builtin_amdgcn_sched_barrier(0);   // many planes: keep the groups' registers apart
-                });
+                }
+            });
             }
             __builtin_amdgcn_sched_barrier(0);   // one pass after the other: keeps the registers of a pass apart
         });
-        if constexpr (OFF && NU > 6 && P == 0) {   // many planes: the offset term in a pass of its own
-            static_for<4 * GSUB>([&](auto G) {
-                constexpr int r = G;
-                float4v xsum = zero4;
-                static_for<SG>([&](auto TT) {
-                    constexpr int t = SG * r + TT;
-                    const half8 xa = *reinterpret_cast<const __attribute__((address_space(3))) half8 *>(xr + t * 16);
-                    xsum = __builtin_amdgcn_mfma_f32_16x16x32_f16(xa, __builtin_bit_cast(half8, ones), xsum, 0, 0, 0);
-                });
-#pragma unroll
-                for (int h = 0; h < 2; h++) {
-                    const float z = scale_of(r, Q, h);
-                    acc[h][0] += z * xsum[0];
-                    acc[h][1] += z * xsum[1];
-                    acc[h][2] += z * xsum[2];
-                    acc[h][3] += z * xsum[3];
-                }
-            });
-        }
         store_activation_row(xrow, xbuf + (cur ^ 1) * kXBufBytes, wave, lane);
         if constexpr (TWO) store_activation_row(xrow2, xbuf + (cur ^ 1) * kXBufBytes, wave + waves, lane);
         __syncthreads();   // the next activation block is in place; this one is no longer read
     }
 
-    // acc[h][v]: activation row 4 kappa + v, output nb * 32 + 16 h + j.  All eight split-k atomics
-    // of a lane are issued before the first answer is looked at.
+    if constexpr (GSUB == 4) {
+        acc[0] = (acc2[0][0] + acc2[0][1]) + acc_off[0];
+        acc[1] = (acc2[1][0] + acc2[1][1]) + acc_off[1];
+    }
+    // acc[h][v] is (activation row j, output nb * 32 + 16 h + 4 kappa + v).  The end of the workgroup
+    // wants the outputs of a row side by side in the lanes (one cache line per row for its stores
+    // and atomics), so each 16 x 16 tile is turned through the wavefront's staging area:
+    // afterwards acc[h][v] is (activation row 4 kappa + v, output nb * 32 + 16 h + j).
+    {
+        __attribute__((address_space(3))) float *turn = reinterpret_cast<__attribute__((address_space(3))) float *>(stage);
+#pragma unroll
+        for (int h = 0; h < 2; h++) {
+            asm volatile("" ::: "memory");   // the reads of the tile before are done with (LDS operations of a wavefront execute in order)
+#pragma unroll
+            for (int v = 0; v < 4; v++) turn[(4 * kappa + v) * 16 + j] = acc[h][v];
+            asm volatile("" ::: "memory");
+            acc[h] = *reinterpret_cast<__attribute__((address_space(3))) float4v *>(turn + j * 16 + 4 * kappa);
+        }
+        asm volatile("" ::: "memory");
+    }
+    // All eight split-k atomics of a lane are issued before the first answer is looked at.
     __half *y = reinterpret_cast<__half *>(a.y);
     bool valid[2][4];
     unsigned long long *word[2][4];

@@ -190,7 +190,7 @@ FusedPlan choose_fused_plan(const Shape *const *shapes, int count, int cus, int 
 // Cost model in microseconds (-1 when `ks` names the same plan as a smaller number of k-splits).
 // A compute unit holds one workgroup.  Per k-block the workgroup spends a fixed time (its
 // wavefronts meet at a barrier) plus a time per wavefront (one tile each); per workgroup a start
-// (launch, pattern table, first memory round trip) and an end (eight split-k atomics per lane: 3 to
+// (launch, first activation block, first memory round trip) and an end (eight split-k atomics per lane: 3 to
 // 5 microseconds of a launch, whatever its shape).  A second round of workgroups costs more than its
 // sum (the units wait for the slowest of a round), so plans that keep all workgroups resident at
 // once win where the shape allows one.  Constants fitted to measured launches of the decoder-layer
@@ -240,7 +240,7 @@ bool batch_kernel_takes(const Shape &s)
 // wavefronts per workgroup and one number of k-blocks per workgroup for all entries.  The grid
 // runs in rounds of one workgroup per compute unit.  A workgroup costs a time per tile (more when
 // every wavefront stages two activation rows), a little per k-block, and a start and end of its own
-// that grows with its wavefronts (pattern table, first tiles, the wait for the slowest wavefront);
+// that grows with its wavefronts (first tiles, the wait for the slowest wavefront);
 // the split-k atomics cost by their number in the whole launch (rows x outputs x k-splits), as
 // the memory side executes them at a fixed rate.  Constants (microseconds) fitted to measured
 // times of 330 plans over eight lists (3 to 12 entries, k and n 2048 to 12288, 1 to 4 planes,

@@ -61,15 +61,14 @@ hipError_t launch_matvec_multi(int q, int has_offset, int gsub, const MultiMatve
 constexpr int kBatchMaxPlanes = 4;
 constexpr int kBatchWaves = 16;
 constexpr int kBatchWavesMin = 8;
-// LDS of a workgroup of the batch kernel: the pattern table (64 KiB), two activation blocks of 17
-// rows of 1040 bytes, and per wavefront a 1 KiB staging area plus the scales of its tile for the
-// matrix lanes (one scale group per 128 k: the lanes' scale words as they are, up to 5; two or four
-// groups per 128 k: 4 bytes per (group, plane or offset, output pair)).  A compute unit has 160 KiB,
-// which bounds the wavefronts of a workgroup when there are four groups per 128 k.
-constexpr int batch_scale_area_bytes(int gsub, int qo) { return gsub == 1 ? 256 * 5 : 256 * gsub * qo; }
+// LDS of a workgroup of the batch kernel: two activation blocks of 17 rows of 2064 bytes (every
+// activation as the pair -x, +x), and per wavefront a 1 KiB staging area plus the scales of its tile
+// for the matrix lanes (64 bytes per (scale group of the k-block, plane or offset)).  A compute
+// unit has 160 KiB, which bounds the wavefronts of a workgroup when there are four groups per 128 k.
+constexpr int batch_scale_area_bytes(int gsub, int qo) { return 256 * gsub * qo; }
 constexpr int batch_lds_bytes(int waves, int gsub, int qo)
 {
-    return 256 * 16 * 16 + 2 * 17 * 1040 + waves * (1024 + batch_scale_area_bytes(gsub, qo));
+    return 2 * 17 * 2064 + waves * (1024 + batch_scale_area_bytes(gsub, qo));
 }
 constexpr int batch_waves_max(int gsub, int qo)
 {

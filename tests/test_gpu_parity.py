@@ -245,18 +245,31 @@ def test_every_launch_plan_agrees(lutgemm, oracle, device):
     W.close()
 
 
+def batch_waves_max(g, qo):
+    """Most wavefronts a workgroup of the batch kernel can have: 160 KiB of LDS hold two activation
+    blocks (17 rows of 2064 bytes each) and per wavefront 1 KiB of staging plus its scale area."""
+    gsub = 1 if g % 128 == 0 else 2 if g % 64 == 0 else 4
+    area = 256 * gsub * qo
+    w = 16
+    while w > 8 and 2 * 17 * 2064 + w * (1024 + area) > 160 * 1024:
+        w -= 1
+    return w
+
+
 @pytest.mark.parametrize("k,n,q,g,offset", [(4096, 520, 2, 128, True), (2048, 200, 3, 64, False), (6144, 97, 1, 32, True),
                                             (8192, 1000, 4, 256, False)])
 def test_every_batch_plan_agrees(lutgemm, oracle, device, k, n, q, g, offset):
-    """The batch kernel under forced launch plans: 8..16 wavefronts per workgroup (fewer than, as
-    many as and more than the batch has rows), one to many k-splits.  Every plan meets the
-    tolerance and repeats bit for bit; a request that cannot be launched is refused."""
+    """The batch kernel under forced launch plans: 8 wavefronts per workgroup up to what the LDS
+    holds (fewer than, as many as and more than the batch has rows), one to many k-splits.  Every
+    plan meets the tolerance and repeats bit for bit; a request that cannot be launched is refused."""
     from lutgemm import synth
     w, W = make(lutgemm, synth, k, n, q, g, offset=offset, seed=k + n)
     ts = (k + 511) // 512
     x = synth.make_x(16, k, seed=n)
     truth = truth_of(oracle, w, x)
+    wmax = batch_waves_max(g, q + (1 if offset else 0))
     for waves, ks in ((8, 1), (12, 2), (16, ts // 2), (10, ts), (16, 2), (14, 1), (9, 2)):
+        waves = min(waves, wmax)
         for m in (8, 5, 3, 12, 16):
             say("case batch plan", k, n, q, g, offset, waves, ks, m)
             W.set_batch_plan(waves, ks)
@@ -265,7 +278,7 @@ def test_every_batch_plan_agrees(lutgemm, oracle, device, k, n, q, g, offset):
             y = run_matvec(lutgemm, W, x[:m], device)
             assert_within_tolerance(y, truth[:m], "m=%d waves=%d ks=%d plan=%s" % (m, waves, ks, bp))
             assert np.array_equal(y.view(np.uint16), run_matvec(lutgemm, W, x[:m], device, cols=True).view(np.uint16))
-    for waves, ks in ((7, 1), (17, 1), (8, ts + 1), (8, 0)):
+    for waves, ks in ((7, 1), (wmax + 1, 1), (8, ts + 1), (8, 0)):
         with pytest.raises(lutgemm.LutGemmError):
             W.set_batch_plan(waves, ks)
     W.set_batch_plan()   # back to the model's choice

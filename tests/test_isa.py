@@ -1,10 +1,12 @@
 """What the compiler made of the batch kernel, checked on the generated gfx950 assembly of the
 library's own translation unit (no GPU needed: hipcc cross-compiles; about a minute).  The hot
 loop and the end of a workgroup depend on properties the source can only ask for: the
-transposition done by the LDS, the matrix instructions present, no packed fp32 forms, and, at the
-end, all answers of the split-k atomics awaited before the first output is stored (a wait behind a
-store also waits for the store's round trip, which cost a launch 1.5 to 2 microseconds when the
-compiler once arranged the code that way)."""
+transposition done by the LDS, the matrix instructions present, the index and the scale
+multiply-add in one instruction each, no packed fp32 forms, no register used while an LDS read
+into it is still in flight (the loop issues its reads ahead through asm statements and waits
+with counts of its own), and, at the end, all answers of the split-k atomics awaited before the
+first output is stored (a wait behind a store also waits for the store's round trip, which cost a
+launch 1.5 to 2 microseconds when the compiler once arranged the code that way)."""
 import os
 import re
 import subprocess
@@ -28,6 +30,56 @@ def kernels_of(tmp_path, source):
     return found
 
 
+def vgprs_named(operand):
+    """VGPR numbers an operand names: v12, v[8:11]"""
+    out = set()
+    for m in re.finditer(r"\bv\[(\d+):(\d+)\]|\bv(\d+)\b", operand):
+        if m.group(3) is not None:
+            out.add(int(m.group(3)))
+        else:
+            out.update(range(int(m.group(1)), int(m.group(2)) + 1))
+    return out
+
+
+def uses_of_registers_in_flight(body):
+    """LDS operations of a wavefront complete in order, and s_waitcnt lgkmcnt(n) returns when at most
+    n are outstanding.  Walks the instructions in program order with that queue (kept across labels
+    and branches, which only makes the check stricter) and returns the instructions that read or
+    write a VGPR while an LDS read into it is queued."""
+    queue, bad = [], []
+    for line in body:
+        line = line.split(";")[0].strip()
+        if not line or line.endswith(":") or line.startswith("."):
+            continue
+        op, _, rest = line.partition(" ")
+        operands = [o.strip() for o in rest.split(",")]
+        if op == "s_waitcnt":
+            m = re.search(r"lgkmcnt\((\d+)\)", rest)
+            if m:
+                n = int(m.group(1))
+                queue = queue[len(queue) - n:] if 0 < n < len(queue) else ([] if n == 0 else queue)
+            continue
+        pending = set().union(*queue) if queue else set()
+        if op.startswith("ds_"):
+            is_read = "read" in op or "load" in op
+            dest = vgprs_named(operands[0]) if is_read else set()
+            sources = set().union(*[vgprs_named(o) for o in (operands[1:] if is_read else operands)])
+            if (sources | dest) & pending:
+                bad.append(line)
+            queue.append(dest)
+        elif set().union(*[vgprs_named(o) for o in operands]) & pending:
+            bad.append(line)
+    return bad
+
+
+def test_the_in_flight_check_sees_a_short_wait():
+    good = ["ds_read_b128 v[0:3], v9", "ds_read_b128 v[4:7], v9 offset:16", "s_waitcnt lgkmcnt(1)", "v_mov_b32_e32 v8, v0",
+            "s_waitcnt lgkmcnt(0)", "v_mov_b32_e32 v8, v4"]
+    assert uses_of_registers_in_flight(good) == []
+    assert uses_of_registers_in_flight([good[0], good[1], "s_waitcnt lgkmcnt(1)", "v_mov_b32_e32 v8, v5"]) == ["v_mov_b32_e32 v8, v5"]
+    assert uses_of_registers_in_flight([good[0], "ds_write_b32 v9, v2"]) == ["ds_write_b32 v9, v2"]
+
+
 def test_batch_kernel_assembly(tmp_path):
     kernels = kernels_of(tmp_path, "batch.hip")
     assert len(kernels) == 48, sorted(kernels)   # 4 plane counts x offset x 3 scale layouts x second staged row
@@ -38,7 +90,12 @@ def test_batch_kernel_assembly(tmp_path):
         assert vgprs <= 128, (name, vgprs)     # 16 wavefronts per workgroup fit a compute unit
         assert ops.count("ds_read_b64_tr_b8") == 4 * q, name            # the transposition is the LDS's
         offset = 1 if "ELb1ELi" in name[:12] else 0
-        assert ops.count("v_mfma_f32_16x16x32_f16") == 32 * q + 16 * offset, name
+        groups_of_32 = "ELi4ELi16E" in name     # four scale groups per 128 k: the scales are the matrix operand, the offset term per output half
+        assert ops.count("v_smfmac_f32_16x16x64_f16") == 32 * q + (32 if groups_of_32 else 16) * offset, name
+        assert ops.count("v_and_or_b32") >= 16 * q, name                  # the index of a step: one instruction per sign word and parity
+        assert "v_cvt_f32_f16_e32" not in ops, name                       # scales applied without conversions
+        assert ops.count("v_fma_mix_f32") >= (0 if groups_of_32 else 32 * q), name
+        assert uses_of_registers_in_flight(body) == [], name
         assert not any(op.startswith(("v_pk_add_f32", "v_pk_mul_f32", "v_pk_fma_f32")) for op in ops), name
         # the end: eight returning atomics, then one wait for all answers, then stores without waits between them
         atomics = [i for i, ln in enumerate(body) if ln.startswith("global_atomic_add_x2") and " sc0" in ln]
