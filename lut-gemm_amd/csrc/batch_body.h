@@ -71,7 +71,6 @@ typedef _Float16 half8 __attribute__((ext_vector_type(8)));
 typedef _Float16 half16 __attribute__((ext_vector_type(16)));
 typedef float float4v __attribute__((ext_vector_type(4)));
 typedef __attribute__((address_space(3))) unsigned char lds_byte;
-typedef uint32_t u32x4v __attribute__((ext_vector_type(4)));
 
 // LDS reads whose order and wait counts are fixed by hand.  The compiler waits for every LDS read
 // right before its first use and schedules that use early, which leaves one read in flight per
@@ -89,9 +88,9 @@ __device__ __forceinline__ half8 lds_read128_at(uint32_t addr)
     return v;
 }
 template <int OFFSET>
-__device__ __forceinline__ u32x4v lds_read128u_at(uint32_t addr)
+__device__ __forceinline__ u32x4 lds_read128u_at(uint32_t addr)
 {
-    u32x4v v;
+    u32x4 v;
     asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(v) : "v"(addr), "n"(OFFSET));
     return v;
 }
@@ -102,7 +101,7 @@ __device__ __forceinline__ void lds_wait(half8 &v)
     asm volatile("s_waitcnt lgkmcnt(%1)" : "+v"(v) : "n"(YOUNGER));
 }
 __device__ __forceinline__ void after_wait(half8 &v) { asm volatile("" : "+v"(v)); }
-__device__ __forceinline__ void after_wait(u32x4v &v) { asm volatile("" : "+v"(v)); }
+__device__ __forceinline__ void after_wait(u32x4 &v) { asm volatile("" : "+v"(v)); }
 __device__ __forceinline__ void after_wait(uint32_t &v) { asm volatile("" : "+v"(v)); }
 template <int OFFSET>
 __device__ __forceinline__ uint32_t lds_read32_at(uint32_t addr)
@@ -264,8 +263,9 @@ __device__ __forceinline__ void batch_workgroup(const MatvecArgs &a, unsigned bl
     // are, [word][lane]; the four words d of lanes 16 G + 4 kappa .. + 3 are the numbers 2 d and 2 d + 1
     // of the lane's four outputs in group G.
     // Two or four groups per 128 k: lane (row r, sub-row sub, jj) holds, in slot t, the scales of
-    // output t SUBL + jj for the group r GSUB + sub; every fp16 number goes (2-byte writes) to
-    // [group][plane or offset][(output % 16) / 4][output half][output % 4].
+    // output t SUBL + jj for the group r GSUB + sub.  Two groups: every fp16 number goes (2-byte
+    // writes) to [group][plane or offset][(output % 16) / 4][output half][output % 4].  Four groups:
+    // the scales are the matrix operand themselves and take a layout of their own (see the loop).
     // (the halves are read back as wider words: the write type may alias them)
     typedef uint16_t __attribute__((may_alias)) aliasing_u16;
     const int s_jj = (lane & 15) % SUBL;
@@ -280,14 +280,14 @@ __device__ __forceinline__ void batch_workgroup(const MatvecArgs &a, unsigned bl
     // LDS byte offset (from saddr) of read number rd (0 .. QO - 1) of group G
     auto scale_read_offset = [](int G, int rd) constexpr { return GSUB == 1 ? rd * 256 + 64 * G : (G * QO + rd) * 64; };
     // acc + scale of (plane or offset B, output half H, output 4 kappa + V) out of the reads of a group * x
-    auto scale_fma = [](float acc, const u32x4v (&reads)[QO], auto Bc, auto Hc, auto Vc, float x) {
+    auto scale_fma = [](float acc, const u32x4 (&reads)[QO], auto Bc, auto Hc, auto Vc, float x) {
         constexpr int B = Bc, H = Hc, V = Vc;
         if constexpr (GSUB == 1) {
             constexpr int hb = H * QO + B;
-            const u32x4v &w = reads[hb >> 1];
+            const u32x4 &w = reads[hb >> 1];
             return fma_half<(hb & 1) != 0>(acc, V == 0 ? w.x : V == 1 ? w.y : V == 2 ? w.z : w.w, x);
         } else {
-            const u32x4v &w = reads[B];
+            const u32x4 &w = reads[B];
             return fma_half<(V & 1) != 0>(acc, H == 0 ? (V < 2 ? w.x : w.y) : (V < 2 ? w.z : w.w), x);
         }
     };
@@ -399,7 +399,7 @@ __device__ __forceinline__ void batch_workgroup(const MatvecArgs &a, unsigned bl
                             after_wait(aw[pair & 1][A]);
                             const uint32_t word = aw[pair & 1][A];
                             const uint32_t lo = __builtin_amdgcn_perm(word, word, 0x01000100u), hi = __builtin_amdgcn_perm(word, word, 0x03020302u);
-                            av[A] = __builtin_bit_cast(half8, u32x4v{lo, lo, hi, hi});
+                            av[A] = __builtin_bit_cast(half8, u32x4{lo, lo, hi, hi});
                         });
                     const half16 xb = __builtin_shufflevector(xb0[slot], xb1[slot], 0, 1, 2, 3, 4, 5, 6, 7, 8, 9, 10, 11, 12, 13, 14, 15);
                     static_for<CH>([&](auto I) {
@@ -430,7 +430,7 @@ __device__ __forceinline__ void batch_workgroup(const MatvecArgs &a, unsigned bl
             };
             constexpr int SR = [&]() constexpr { int c = 0; for (int rd = 0; rd < QO; rd++) c += needed(rd) ? 1 : 0; return c; }();   // scale reads with the last step of a group
             half8 xb0[P + 1], xb1[P + 1];
-            u32x4v sw[2][QO];
+            u32x4 sw[2][QO];
             float4v part[CH];
             float4v xsum = zero4;
             auto issue = [&](auto Gc) {
