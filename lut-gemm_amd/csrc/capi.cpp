@@ -184,48 +184,40 @@ FusedPlan choose_fused_plan(const Shape *const *shapes, int count, int cus, int 
 }
 
 // Launch plan of the batch kernel (3..16 rows per pass on the matrix cores): wavefronts per
-// workgroup and k-splits.  The kernel is bound on the compute units (matrix and vector instruction
-// issue, expansion of the sign bytes through LDS), not by the stream, so what matters is an even
-// spread of the tiles over the compute units.
+// workgroup and k-splits.  The kernel is bound on the compute units, not by the stream, so what
+// matters is an even spread of the tiles over the compute units.
 // Cost model in microseconds (-1 when `ks` names the same plan as a smaller number of k-splits).
-// A compute unit holds one workgroup.  Per k-block the workgroup spends a fixed time (its
-// wavefronts meet at a barrier) plus a time per wavefront (one tile each); per workgroup a start
-// (launch, first activation block, first memory round trip) and an end (eight split-k atomics per lane: 3 to
-// 5 microseconds of a launch, whatever its shape).  A second round of workgroups costs more than its
-// sum (the units wait for the slowest of a round), so plans that keep all workgroups resident at
-// once win where the shape allows one.  Constants fitted to measured launches of the decoder-layer
-// shapes (k = 12288 or 49152, n = 12288 .. 49152, two planes, eight rows).
-double batch_plan_cost(const Shape &s, int cus, int waves, int ks, Plan *out)
+// A compute unit holds one workgroup, so the grid runs in rounds of one workgroup per unit.  A
+// workgroup costs a time per tile (wavefronts x k-blocks x planes) and a start and end of its own;
+// the split-k atomics cost by their number in the whole launch (rows x outputs x k-splits: the
+// memory side executes them at a fixed rate).  Constants fitted to 190 measured plans over eight
+// shapes (k and n 4096 to 49152, two to four planes, eight rows; rms error 7 %); the fit names the
+// fastest measured plan of every shape.
+double batch_plan_cost(const Shape &s, int cus, int waves, int ks, int rows, Plan *out)
 {
-    const double tile_us = 0.0635 * s.q, block_us = 1.82, start_us = 11.4, round_us = 8.0;
+    const double tile_us = 0.1123 * s.q, group_us = 4.95, atomic_us = 7.08e-6;
     const int ntiles = div_up(s.nb, waves);
     const int bps = div_up(s.ts, ks);
     if (div_up(s.ts, bps) != ks) return -1.0;
     const long wgs = (long)ntiles * ks;
     const int rounds = (int)((wgs + cus - 1) / cus);
     *out = Plan{waves, ntiles, bps, ks};
-    return rounds * (bps * (waves * tile_us + block_us) + start_us) + (rounds - 1) * round_us + 0.02 * ks;
+    return rounds * (bps * waves * tile_us + group_us) + (ks > 1 ? atomic_us * (double)s.n * rows * ks : 0.0);
 }
 
-Plan choose_batch_plan(const Shape &s, int cus)
+// `rows`: 8 for passes of up to 8 rows, 16 for larger ones (the two plans a handle keeps)
+Plan choose_batch_plan(const Shape &s, int cus, int rows)
 {
     const int wmax = lutgemm_kernels::batch_waves_max(s.gsub, s.qo), wmin = lutgemm_kernels::kBatchWavesMin;
     Plan best{wmax, div_up(s.nb, wmax), s.ts, 1};
     double best_cost = 1e30;
-    long best_wgs = 0;
     for (int waves = wmin; waves <= wmax; waves++)
         for (int ks = 1; ks <= s.ts && ks <= kMaxSplits; ks++) {
             Plan p;
-            const double cost = batch_plan_cost(s, cus, waves, ks, &p);
-            if (cost < 0.0) continue;
-            const long wgs = (long)p.ntiles * p.k_splits;
-            // plans the model puts within 4 % of each other: the one that keeps more compute
-            // units busy in a single round has measured better
-            const bool tie = wgs <= cus && best_wgs <= cus && cost < best_cost * 1.04 && cost > best_cost * 0.96;
-            if (tie ? wgs > best_wgs : cost < best_cost) {
-                if (cost < best_cost) best_cost = cost;
+            const double cost = batch_plan_cost(s, cus, waves, ks, rows, &p);
+            if (cost >= 0.0 && cost < best_cost) {
+                best_cost = cost;
                 best = p;
-                best_wgs = wgs;
             }
         }
     return best;
@@ -568,7 +560,7 @@ int run_matvec(const lutgemm_weight *w, const void *x, void *y, int m, void *str
         // up to 16 rows per pass over the weight on the matrix cores
         const int pass_rows = m < kRowsPerPass ? m : kRowsPerPass;
         const Plan plan = w->batch_measured[pass_rows > 8] ? w->plan_batch[pass_rows > 8]
-                                                            : choose_batch_plan(s, w->compute_units);
+                                                            : choose_batch_plan(s, w->compute_units, pass_rows > 8 ? kRowsPerPass : 8);
         a.ntiles = plan.ntiles;
         a.k_splits = plan.k_splits;
         a.blocks_per_split = plan.blocks_per_split;
@@ -992,7 +984,8 @@ int lutgemm_weight_plan_for(const lutgemm_weight *w, int m, int *workgroups, int
     Plan p = m == 1 ? w->plan : w->plan2;
     if (m >= 3 && batch_kernel_takes(w->shape)) {
         const int pass_rows = m < kRowsPerPass ? m : kRowsPerPass;
-        p = w->batch_measured[pass_rows > 8] ? w->plan_batch[pass_rows > 8] : choose_batch_plan(w->shape, w->compute_units);
+        p = w->batch_measured[pass_rows > 8] ? w->plan_batch[pass_rows > 8]
+                                              : choose_batch_plan(w->shape, w->compute_units, pass_rows > 8 ? kRowsPerPass : 8);
     }
     if (workgroups) *workgroups = p.ntiles * p.k_splits;
     if (waves_per_group) *waves_per_group = p.waves;
@@ -1019,7 +1012,7 @@ int lutgemm_weight_set_batch_plan(lutgemm_weight *w, int waves_per_group, int k_
     if (k_splits < 1 || k_splits > s.ts || k_splits > kMaxSplits)
         return fail(LUTGEMM_ERR_BAD_SHAPE, "k_splits=%d outside 1..%d", k_splits, s.ts < kMaxSplits ? s.ts : kMaxSplits);
     Plan p;
-    if (batch_plan_cost(s, w->compute_units, waves_per_group, k_splits, &p) < 0.0)
+    if (batch_plan_cost(s, w->compute_units, waves_per_group, k_splits, 8, &p) < 0.0)
         return fail(LUTGEMM_ERR_BAD_SHAPE, "k_splits=%d leaves a k-split without k-blocks (%d k-blocks)", k_splits, s.ts);
     w->plan_batch[0] = w->plan_batch[1] = p;
     w->batch_measured[0] = w->batch_measured[1] = true;
@@ -1189,7 +1182,7 @@ int lutgemm_weight_autotune(lutgemm_weight *w, void *stream)
         for (int waves = lutgemm_kernels::kBatchWavesMin; waves <= lutgemm_kernels::batch_waves_max(s.gsub, s.qo); waves++)
             for (int ks = 1; ks <= s.ts && ks <= kMaxSplits; ks++) {
                 Plan p;
-                const double cost = batch_plan_cost(s, w->compute_units, waves, ks, &p);
+                const double cost = batch_plan_cost(s, w->compute_units, waves, ks, rows, &p);
                 if (cost >= 0.0) timed.push_back(Timed{1e30f, cost, p});
             }
         std::sort(timed.begin(), timed.end(), [](const Timed &a, const Timed &b) { return a.cost < b.cost; });
