@@ -578,6 +578,39 @@ def test_matvec_many_fuses_batches(lutgemm, oracle, device):
         W.close()
 
 
+@pytest.mark.parametrize("q,g,offset", [(2, 32, True), (4, 32, False), (3, 64, True), (4, 128, True), (1, 96, False)])
+def test_matvec_many_fuses_batches_of_every_scale_layout(lutgemm, oracle, device, q, g, offset):
+    """Fused batches with four, two and one scale group per 128 k (with groups of 32 k the scales
+    are the matrix operand), with and without the offset term, ragged shapes, 3 to 16 rows: every
+    entry meets the tolerance and the call repeats bit for bit."""
+    import torch
+    from lutgemm import synth
+    st = torch.cuda.current_stream().cuda_stream
+    shapes = [(1536, 520), (2304, 1000), (768, 96)] if g == 96 else [(1536, 520), (2048, 1000), (1024, 96)]
+    rows = [8, 3, 16]
+    ws = [make(lutgemm, synth, k, n, q, g, offset=offset, seed=300 + i + q) for i, (k, n) in enumerate(shapes)]
+    xh = [synth.make_x(m, k, seed=k + m) for (k, _), m in zip(shapes, rows)]
+    xs = [torch.from_numpy(v).to(device) for v in xh]
+    ys = [torch.full((m, W.mSize), float("nan"), dtype=torch.float16, device=device) for (_, W), m in zip(ws, rows)]
+    seq = lutgemm.MatvecSequence([(W, x.data_ptr(), y.data_ptr(), m) for (_, W), x, y, m in zip(ws, xs, ys, rows)])
+    first = None
+    for rep in range(2):
+        for y in ys:
+            y.fill_(float("nan"))
+        say("case fused batches", q, g, offset, "rep", rep)
+        seq.launch(st)
+        torch.cuda.synchronize()
+        got = [y.clone() for y in ys]
+        if first is None:
+            first = got
+            for (w, _), x, y, m in zip(ws, xh, got, rows):
+                assert_within_tolerance(y.cpu().numpy(), truth_of(oracle, w, x), "q=%d g=%d m=%d" % (q, g, m))
+        else:
+            assert all(torch.equal(a.view(torch.int16), b.view(torch.int16)) for a, b in zip(first, got))
+    for _, W in ws:
+        W.close()
+
+
 def test_matvec_many_fuses_two_row_entries(lutgemm, oracle, device):
     """Independent entries of two rows share one launch of the two-row table-lookup kernel (any
     number of planes; runs are cut where planes, offset or the scale layout change and where a
