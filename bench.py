@@ -6,8 +6,12 @@
 Default (cfg1, the headline): a step is one matvec of m=1, k=n=12288, q=3, g=128, fp16
 activations, no offset, with the packed weight already resident in HBM.  Consecutive steps use
 different weight copies (R copies, R * packed bytes > 4 x the 256 MiB last-level cache), so every
-step streams its weight from HBM and not from cache.  The K timed steps are issued back to back
-with one C-ABI call and bracketed by HIP events on the launch stream.
+step streams its weight from HBM and not from cache.  The K timed steps are issued back to back,
+ONE KERNEL LAUNCH PER MATVEC (the protocol of the reference's own caller, a loop of lutGEMM::matmul
+calls, tests/opt/fp16/int3_col_wise_matmul_fp16.cu:120-133), and bracketed by HIP events on the
+launch stream: that is `value`, `ms_per_step` and `roofline.frac`.  The same steps as independent
+matvecs sharing launches (lutgemm_matvec_many) are reported beside it (`fused_independent`, and
+`roofline.frac_fused_independent`).
 
 Prints ONE JSON line: value = packed-weight GB/s (higher is better), plus us per matvec, the
 roofline block for the matvec kernel, the dense fp16 GEMV comparator, the single-copy ("hot")
@@ -38,11 +42,13 @@ for _p in (ROOT, os.path.join(ROOT, "lut-gemm_amd")):
 HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published peak
 LLC_BYTES = 256 << 20  # last-level (memory-side) cache
 METRIC = "µs/matvec + weight-GB/s (% HBM peak), n=k=12288 q=3 g=128 m=1 fp16"
-# HBM bytes per cfg1 matvec inside a launch of lutgemm_matvec_many, from the rocprofv3 counter runs
-# summarised in profiles/lut_matvec_multi_kernel_cfg1.md (FETCH_SIZE and WRITE_SIZE per dispatch,
-# scaled by the factors a plain copy kernel of known size reads on the same counters, divided by
-# the matvecs of the dispatch): 63.72 MB read + 0.32 MB written
-CFG1_MEASURED_TRAFFIC_BYTES_PER_MATVEC = 64.04e6
+# HBM bytes per launch of lut_matvec_kernel<3,false,1> on cfg1 with the launch plan 8 wavefronts x 5
+# k-splits, from the rocprofv3 counter runs summarised in profiles/lut_matvec_kernel_cfg1.md
+# (FETCH_SIZE x 2.000 + WRITE_SIZE x 1.000 per dispatch, the factors a plain copy kernel of known
+# size reads on the same counters): 64.01 MB read + 0.61 MB written.  Quoted only when the run
+# uses that plan; any other launch shape reports null.
+CFG1_PROFILED_PLAN = (8, 5)
+CFG1_PROFILED_TRAFFIC_BYTES_PER_LAUNCH = 64.62e6
 
 
 def event_time_ms(torch, fn, stream):
@@ -207,7 +213,7 @@ def time_point(lutgemm, torch, stream, pt, steps, warmup):
     steps, then (whatever `warmup` is) PREWARM_MS of launches so that the clocks are up, then
     BURSTS bursts of exactly `steps` steps; the median burst counts.  The rotation over the weight
     copies continues from burst to burst, so no burst finds its weights in the memory-side cache.
-    pt.fused_us: the same bursts through lutgemm_matvec_many, which puts up to sixteen independent
+    pt.fused_us: the same bursts through lutgemm_matvec_many, which puts up to 32 independent
     matvecs (here: different weight copies) into one launch."""
     sh = stream.cuda_stream
     lutgemm.MatvecSequence(pt.items(max(1, warmup))).launch(sh, fused=False)
@@ -255,8 +261,8 @@ def run_single(args, lutgemm, synth, torch, dev, stream, name):
     k, n, q, g = cfg["k"], cfg["n"], cfg["q"], cfg["g"]
     pt = Point(lutgemm, synth, torch, dev, k, n, q, g, cfg["rtn"], 1, 1, stream.cuda_stream,
                copies=args.copies if name == "cfg1" else None, plan=args.plan)
-    us_each, us_hot = time_point(lutgemm, torch, stream, pt, args.steps, args.warmup)
-    us = pt.fused_us     # the steps are independent matvecs: whole-job throughput through lutgemm_matvec_many
+    us, us_hot = time_point(lutgemm, torch, stream, pt, args.steps, args.warmup)
+    us_fused = pt.fused_us
     weight_gbs = pt.b_w / (us * 1e-6) / 1e9
     achieved = pt.b_total / (us * 1e-6) / 1e9
     parity, truth = pt.parity(None if name != "cfg2" else 4096)
@@ -267,30 +273,37 @@ def run_single(args, lutgemm, synth, torch, dev, stream, name):
     units = min(args.steps, MAX_FUSED, pt.copies)
     line = base_line(args, metric, weight_gbs, us, workload,
                      {"weight_copies_rotated": pt.copies, "packed_weight_bytes": pt.b_w,
-                      "launch": "the %d steps of a burst are independent matvecs (one weight copy each) issued with one "
-                                "lutgemm_matvec_many call, which puts up to %d of them into one kernel launch" % (args.steps, MAX_FUSED),
-                      "plan_of_single_launches": pt.plan})
+                      "launch": "one kernel launch per matvec (lutgemm_matvec_each), %d launches back to back per timed burst, "
+                                "every launch on its own copy of the weight: what a chain of matvecs that depend on each other "
+                                "sees, and the protocol of the reference's caller" % args.steps,
+                      "plan": pt.plan})
     line["ms_per_step"] = us / 1e3
-    kernel = "lut_matvec_multi_kernel<%d,%s,1>" % (q, "true" if pt.has_offset else "false")
-    traffic_unit = CFG1_MEASURED_TRAFFIC_BYTES_PER_MATVEC if name == "cfg1" else None
+    tag = "%d,%s,1" % (q, "true" if pt.has_offset else "false")
+    profiled = name == "cfg1" and (pt.plan["waves"], pt.plan["k_splits"]) == CFG1_PROFILED_PLAN
     line["roofline"] = {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                         "frac": achieved / HBM_PEAK_GBS,
-                        "traffic": traffic_unit * units if traffic_unit is not None else None,
+                        "traffic": CFG1_PROFILED_TRAFFIC_BYTES_PER_LAUNCH if profiled else None,
                         "traffic_source": (
-                            "not measured in this run: rocprofv3 --pmc FETCH_SIZE x 2.000 + WRITE_SIZE x 1.000 per dispatch of "
-                            "this kernel divided by the matvecs of the dispatch, from profiles/lut_matvec_multi_kernel_cfg1.md, "
-                            "times the matvecs per launch of this run" if traffic_unit is not None else
-                            "no counter run on record for this workload (profiles/)"),
-                        "kernel": kernel, "matvecs_per_launch": units,
-                        "algorithmic_bytes_per_launch": pt.b_total * units, "avg_launch_us": us * units,
-                        "us_per_matvec_bursts": pt.fused_burst_us}
-    line["one_launch_per_matvec"] = {
-        "what": "the same bursts with one kernel launch per matvec (lutgemm_matvec_each): what a chain of matvecs that "
-                "depend on each other sees; every launch pays its own start, end and launch gap",
-        "kernel": "lut_matvec_kernel<%d,%s,1>" % (q, "true" if pt.has_offset else "false"), "plan": pt.plan,
-        "us_per_matvec": us_each, "weight_GBps": pt.b_w / us_each / 1e3,
-        "roofline_frac": pt.b_total / us_each / 1e3 / HBM_PEAK_GBS, "us_per_matvec_bursts": pt.burst_us,
-        "hot_single_copy_us_per_matvec": us_hot}
+                            "not measured in this run: rocprofv3 --pmc FETCH_SIZE x 2.000 + WRITE_SIZE x 1.000 per dispatch of this "
+                            "kernel with this launch plan, from profiles/lut_matvec_kernel_cfg1.md" if profiled else
+                            "null: no counter run on record for this kernel with this launch plan (profiles/)"),
+                        "kernel": "lut_matvec_kernel<%s>" % tag, "matvecs_per_launch": 1,
+                        "algorithmic_bytes_per_launch": pt.b_total, "avg_launch_us": us,
+                        "us_per_matvec_bursts": pt.burst_us,
+                        "value_is": "back_to_back",
+                        "frac_back_to_back": achieved / HBM_PEAK_GBS, "us_back_to_back": us,
+                        "frac_fused_independent": pt.b_total / us_fused / 1e3 / HBM_PEAK_GBS,
+                        "us_fused_independent": us_fused,
+                        "hot_single_copy_us_per_matvec": us_hot}
+    line["fused_independent"] = {
+        "what": "the same bursts as INDEPENDENT matvecs through lutgemm_matvec_many, which puts up to %d of them (own weight "
+                "copy each) into one kernel launch; not what dependent matvecs get" % MAX_FUSED,
+        "kernel": "lut_matvec_multi_kernel<%s>" % tag, "matvecs_per_launch": units,
+        "us_per_matvec": us_fused, "weight_GBps": pt.b_w / us_fused / 1e3,
+        "roofline_frac": pt.b_total / us_fused / 1e3 / HBM_PEAK_GBS,
+        "algorithmic_bytes_per_launch": pt.b_total * units, "avg_launch_us": us_fused * units,
+        "us_per_matvec_bursts": pt.fused_burst_us}
+    us_each = us
     # the device's pure-read time for the same tiles, same grid, same rotation over the copies,
     # timed like the matvec (clocks warmed, median of BURSTS bursts)
     reads = max(1, args.steps)
@@ -299,7 +312,7 @@ def run_single(args, lutgemm, synth, torch, dev, stream, name):
     rms = time_bursts(torch, stream, [(lambda o=o: lutgemm.read_probe(o, stream.cuda_stream)) for o in orders])
     read_us = median(rms) * 1e3 / reads
     tile_bytes = sum(lutgemm.packed_sizes(k, n, q, k // g, pt.has_offset))  # packed tiles incl. padding
-    line["one_launch_per_matvec"]["pure_read_same_tiles"] = {
+    line["pure_read_same_tiles"] = {
         "what": "one launch per weight that only reads the tiles (same grid, same loads in flight): the floor of a single launch",
         "us": read_us, "bytes": tile_bytes, "GBps": tile_bytes / read_us / 1e3, "matvec_time_over_read_time": us_each / read_us}
     line["roofline"]["read_floor_us_single_launch"] = read_us
@@ -337,7 +350,7 @@ def run_single(args, lutgemm, synth, torch, dev, stream, name):
         dense = {"kind": "torch.mv fp16 (rocBLAS/hipBLASLt)", "us_per_matvec": dense_us,
                  "bytes": 2 * k * n + 2 * k + 2 * n,
                  "GBps": (2 * k * n + 2 * k + 2 * n) / (dense_us * 1e-6) / 1e9,
-                 "lut_speedup": dense_us / us, "lut_speedup_one_launch_per_matvec": dense_us / us_each}
+                 "lut_speedup": dense_us / us, "lut_speedup_fused_independent": dense_us / us_fused}
         # the same product through this library's plain streaming kernel (bandwidth-bound comparator)
         sh = stream.cuda_stream
         for i in range(10):
@@ -350,7 +363,7 @@ def run_single(args, lutgemm, synth, torch, dev, stream, name):
                 lutgemm.dense_gemv(Wd[i % nd].data_ptr(), xv.data_ptr(), outs[i % nd].data_ptr(), k, n, sh)
         pus = event_time_ms(torch, run_plain, stream) * 1e3 / reps
         dense["handwritten_streaming_gemv"] = {"us_per_matvec": pus, "GBps": dense["bytes"] / pus / 1e3,
-                                                "lut_speedup": pus / us, "lut_speedup_one_launch_per_matvec": pus / us_each,
+                                                "lut_speedup": pus / us, "lut_speedup_fused_independent": pus / us_fused,
                                                 "agrees_with_library": agree}
         del Wd
     line["dense_fp16_gemv"] = dense
@@ -388,18 +401,21 @@ def run_cfg3(args, lutgemm, synth, torch, dev, stream):
         tot_us += us
         tot_fused += pt.fused_us
         pt.close()
-    value = tot_bytes / tot_fused / 1e3
+    value = tot_bytes / tot_us / 1e3
+    fused = tot_bytes / tot_fused / 1e3
     line = base_line(args, "weight-GB/s over the k=n=7168 sweep (q 1..4 x g 32,64,128,k), m=1 fp16", value,
-                     tot_fused / len(points), "cfg3: 16 BCQ matvecs k=n=7168, q in 1..4, g in {32,64,128,7168}",
+                     tot_us / len(points), "cfg3: 16 BCQ matvecs k=n=7168, q in 1..4, g in {32,64,128,7168}",
                      {"points": len(points),
-                      "launch": "per point, bursts of independent matvecs (one weight copy each) through lutgemm_matvec_many"})
-    line["ms_per_step"] = tot_fused / 1e3
+                      "launch": "per point, bursts with one kernel launch per matvec (one weight copy each), back to back"})
+    line["ms_per_step"] = tot_us / 1e3
     line["points"] = points
-    line["one_launch_per_matvec"] = {"weight_GBps": tot_bytes / tot_us / 1e3, "us_sum": tot_us,
-                                     "frac_hbm_peak": tot_bytes / tot_us / 1e3 / HBM_PEAK_GBS}
+    line["fused_independent"] = {"weight_GBps": fused, "us_sum": tot_fused, "frac_hbm_peak": fused / HBM_PEAK_GBS,
+                                 "what": "the same bursts as independent matvecs through lutgemm_matvec_many"}
     line["parity"] = {"worst_max_abs": worst, "outputs_checked_per_point": 2048}
     line["roofline"] = {"bound": "hbm", "achieved": value, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                        "frac": value / HBM_PEAK_GBS, "traffic": None, "kernel": "lut_matvec_multi_kernel<q,false,gsub>",
+                        "frac": value / HBM_PEAK_GBS, "traffic": None, "kernel": "lut_matvec_kernel<q,false,gsub>",
+                        "value_is": "back_to_back", "frac_back_to_back": value / HBM_PEAK_GBS,
+                        "frac_fused_independent": fused / HBM_PEAK_GBS,
                         "note": "aggregate packed-weight bytes / summed time over the 16 points"}
     line["cpu_baseline"] = None
     return line

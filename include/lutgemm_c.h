@@ -39,7 +39,8 @@ typedef enum lutgemm_status {
 } lutgemm_status;
 
 /* Opaque packed weight: device-resident sign tiles, scales and offsets plus the launch plan
- * and the split-k accumulators (64-bit words, two per output and launching stream).  Stands in for class lutGEMM::nQWeight_fp16
+ * and the workspace of the launching streams (split-k accumulators: 64-bit words, one per output and
+ * activation row of a pass; staging rows of the column-batched form).  Stands in for class lutGEMM::nQWeight_fp16
  * (lutGEMM/include/nQWeight_fp16.h:27-52). */
 typedef struct lutgemm_weight lutgemm_weight;
 
@@ -55,7 +56,8 @@ typedef struct lutgemm_weight_info_t {
     size_t sign_bytes;   /* k*n*q/8: packed sign bytes streamed per matvec (unpadded) */
     size_t scale_bytes;  /* num_groups*q*n*2 (unpadded) */
     size_t offset_bytes; /* num_groups*n*2 or 0 (unpadded) */
-    size_t device_bytes; /* bytes of device memory held by the handle, workspace included */
+    size_t device_bytes; /* bytes of device memory held by the handle: tiles, split-k accumulators and
+                            staging rows of every stream set allocated so far */
 } lutgemm_weight_info_t;
 
 /* Build a packed weight from HOST arrays in the layout above (floats are rounded to fp16,
@@ -90,15 +92,21 @@ int lutgemm_weight_info(const lutgemm_weight *w, lutgemm_weight_info_t *info);
  * 1 <= m <= LUTGEMM_MAX_BATCH streams the packed weight: m == 1 and m == 2 through the table-lookup
  * kernels (a two-row pass gives each row bit-identical to its own one-row call), m >= 3 through
  * the batch kernel, which takes up to 16 rows per pass over the weight and contracts them on the
- * matrix cores while a tile is in registers (group sizes that are multiples of 128; other group
- * sizes take table-lookup passes of two rows).  Batch results are deterministic and within the
- * same tolerance, but a row may differ in the last bit from its own one-row call (another order
+ * matrix cores while a tile is in registers (weights of up to four planes, any group size; weights
+ * of more planes take table-lookup passes of two rows).  Batch results are deterministic and within
+ * the same tolerance, but a row may differ in the last bit from its own one-row call (another order
  * of the fp32 additions).
- * Launches on one stream run one after the other and share the handle's split-k accumulators;
- * every further stream that launches on the handle gets accumulators of its own (four streams
- * per handle, LUTGEMM_ERR_UNSUPPORTED beyond; lutgemm_weight_reset_workspace releases them), so
- * launches on different streams may overlap in time.  Launches from different host threads on the
- * SAME stream must be serialised by the caller, as for any stream.
+ * Launches on one stream run one after the other and share one set of split-k accumulators of the
+ * handle; every further stream that launches on the handle gets a set of its own (allocated at that
+ * stream's first launch, so not under graph capture), so launches on different streams may overlap
+ * in time.  A handle keeps four sets.  A fifth stream takes over the set of the stream that used
+ * the handle least recently: at once if that stream's launches on the handle have completed,
+ * otherwise the new stream is made to wait for them (hipStreamWaitEvent) first; to know, every
+ * launch records an event once a handle serves more than one stream.  Launches issued under graph
+ * capture are not tracked, and a set last used that way is never handed on
+ * (LUTGEMM_ERR_UNSUPPORTED if no set can be taken over; lutgemm_weight_clone gives further streams
+ * handles of their own).  Launches from different host threads on the SAME stream must be serialised
+ * by the caller, as for any stream.
  * Non-finite values follow IEEE arithmetic whatever the launch plan: a NaN activation gives NaN
  * outputs, infinite partial sums give an infinity of their sign, or NaN if both signs occur.  With
  * more than one k-split the partial sums are added as fixed-point integers (2^-24 resolution);
@@ -122,9 +130,9 @@ int lutgemm_matvec_static(const lutgemm_weight *w, const void *x, void *y, int m
 /* Column-batched form: x is [k][m] and y is [n][m] (m vectors stored as columns).
  * Replaces lutGEMM::matmul(void* output, nQWeight_fp16&, void* input, int n, int algo)
  * (lutGEMM/include/kernels.h:26, lutGEMM/src/kernels.cu:56-63).  For m == 1 it is the same
- * operation as lutgemm_matvec.  For m > 1 the columns are first gathered into a staging buffer
- * owned by the handle (one per launching stream).  Up to m = 16 nothing is allocated; a larger m
- * grows the buffer the first time it occurs (device synchronisation, free and allocation). */
+ * operation as lutgemm_matvec.  For m > 1 the columns are first gathered into staging rows owned
+ * by the handle (one buffer per launching stream).  Up to m = 16 nothing is allocated; a larger m
+ * grows the stream's buffer the first time it occurs (synchronises that stream, frees, allocates). */
 int lutgemm_matvec_cols(const lutgemm_weight *w, const void *x, void *y, int m, void *stream);
 
 /* `count` matvecs with a single call (a decoder layer's projections, a benchmark loop): entry i
@@ -150,7 +158,8 @@ int lutgemm_matvec_each(const lutgemm_weight *const *ws, const void *const *xs, 
                         const int *ms, int count, void *stream);
 
 /* Put every split-k accumulator of the handle back to zero and forget which streams have
- * launched on it (synchronises the device, then runs a fill kernel on `stream` and waits for it).
+ * launched on it (synchronises the device, then runs fill kernels on `stream` and waits for them;
+ * allocated sets stay allocated).
  * Only needed after a launch was aborted half way (a failed launch in the middle of a batched call,
  * a device fault): completed launches always leave their accumulators at zero.  No counterpart in
  * the reference, which clears its output with cudaMemset before every call
@@ -197,9 +206,10 @@ int lutgemm_weight_plan(const lutgemm_weight *w, int *workgroups, int *waves_per
 int lutgemm_weight_plan_for(const lutgemm_weight *w, int m, int *workgroups, int *waves_per_group,
                             int *k_splits, int *k_blocks_per_group);
 
-/* Override the launch plan, for one-row and two-row launches alike (0 keeps the automatic
- * choice for that field); synchronises the device first.  Returns LUTGEMM_ERR_BAD_SHAPE if the request cannot be launched
- * (1..12 waves per workgroup, 1..min(k/512 rounded up, 128) k-splits). */
+/* Override the launch plan of the table-lookup kernels, for one-row and two-row launches alike (0
+ * keeps the automatic choice for that field; the batch kernel has lutgemm_weight_set_batch_plan);
+ * synchronises the device first.  Returns LUTGEMM_ERR_BAD_SHAPE if the request cannot be launched
+ * (1..12 wavefronts per workgroup, 1..min(k/512 rounded up, 128) k-splits). */
 int lutgemm_weight_set_plan(lutgemm_weight *w, int waves_per_group, int k_splits);
 
 /* Override the batch kernel's launch plan (calls with 3 or more rows on weights of up to four

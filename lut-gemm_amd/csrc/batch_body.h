@@ -122,10 +122,6 @@ __device__ __forceinline__ float fma_half(float acc, uint32_t pair, float x)
     return __builtin_fmaf((float)(HIGH ? h.y : h.x), x, acc);
 }
 
-#ifndef LUTGEMM_BATCH_AHEAD
-#define LUTGEMM_BATCH_AHEAD 1
-#endif
-
 // One activation row of a k-block in LDS: 64 chunks x 2 parities x 16 bytes, block (c, p) at
 // 16 * (16 (c % 8) + 2 (c / 8) + p), and 16 bytes of padding: the B lanes of one read differ in
 // row and in c % 8 only, so the 16 lanes the LDS serves together fall into 16 different 16-byte
@@ -361,7 +357,7 @@ __device__ __forceinline__ void batch_workgroup(const MatvecArgs &a, unsigned bl
             });
             // Steps g = 4 w + 2 hh + p of the k-block.  The LDS reads of step g + P are issued before
             // step g is waited for and contracted.
-            constexpr int P = LUTGEMM_BATCH_AHEAD;
+            constexpr int P = 1;
             constexpr bool WITH_OFFSET4 = OFF && C == 0;
             const uint32_t xaddr = (uint32_t)(size_t)xr;
             if constexpr (GSUB == 4) {

@@ -5,6 +5,7 @@
 #include <hip/hip_runtime_api.h>
 
 #include <algorithm>
+#include <atomic>
 #include <chrono>
 #include <cmath>
 #include <cstdarg>
@@ -57,24 +58,34 @@ struct Plan {
 
 }  // namespace
 
+// What the launches of one stream on a handle share.  Launches on one stream run one after the other;
+// every other stream that launches on the handle gets a set of its own, so launches that overlap on
+// different streams never touch the same words.  Set 0 exists from creation (so a handle used from one
+// stream never allocates in a launch call); further sets are allocated when a further stream first
+// launches.  With all sets taken, a new stream takes over the least recently used set whose latest
+// launch has completed (or, if none has, waits for the least recently used one's): for that, every
+// launch records the set's event once the handle serves more than one stream.
+struct StreamSet {
+    void *stream;                // the stream the set serves
+    unsigned long long *accum;   // rows_per_set x (padded outputs) split-k words, zero between launches
+    void *xrows;                 // staging of column-batched activations: xrows_cols rows of k halves,
+    int xrows_cols;              //   grown on demand
+    hipEvent_t done;             // recorded behind the set's latest launch (only while done_valid)
+    bool done_valid;
+    unsigned long long last_use;
+};
+
 struct lutgemm_weight {
     Shape shape;
     int device;
     int compute_units;
     uint8_t *d_signs;
     uint16_t *d_scales;
-    // Split-k accumulators: kStreamSlots sets of kRowsPerPass x (padded outputs) 64-bit words.
-    // Launches on one stream run one after the other and share a set; every other stream that
-    // launches on this handle gets a set of its own, so launches that overlap on different
-    // streams never touch the same words.
-    unsigned long long *d_accum;
-    size_t accum_bytes;
-    size_t slot_words;
+    int rows_per_set;             // activation rows a launch on this weight can take: 16 (batch kernel) or 2
     std::mutex slot_mutex;
-    void *slot_stream[kStreamSlots];
-    int slots_used;
-    void *d_xrows;                // staging for column-batched activations: per stream set
-    int xrows_cols;               //   xrows_cols rows of k halves; grown on demand beyond that
+    StreamSet set[kStreamSlots];
+    int slots_used;               // sets that serve a stream
+    unsigned long long use_clock;
     Plan plan;                    // launches with one activation row
     Plan plan2;                   // passes over two activation rows (m >= 2): same k-split as plan
     // Batch kernel (3 or more rows): measured plans for passes of up to 8 rows [0] and of 9..16 rows
@@ -286,45 +297,116 @@ int check_device(const lutgemm_weight *w)
     return LUTGEMM_OK;
 }
 
-int alloc_workspace(lutgemm_weight *w)
+size_t set_words(const lutgemm_weight *w) { return (size_t)w->rows_per_set * w->shape.nb * kBatch; }
+
+// Device memory of set i (idempotent).  Allocates: not for a stream that is being captured.
+int alloc_set(lutgemm_weight *w, int i)
 {
-    if (w->d_accum) return LUTGEMM_OK;  // size depends on the shape only
-    w->slot_words = (size_t)kRowsPerPass * w->shape.nb * kBatch;
-    w->accum_bytes = (size_t)kStreamSlots * w->slot_words * sizeof(unsigned long long);
-    hipError_t e = hipMalloc((void **)&w->d_accum, w->accum_bytes);
-    if (e != hipSuccess) return hip_fail(e, "hipMalloc(split-k accumulators)");
-    e = hipMemset(w->d_accum, 0, w->accum_bytes);
-    if (e != hipSuccess) return hip_fail(e, "hipMemset(split-k accumulators)");
-    e = hipMalloc(&w->d_xrows, (size_t)kStreamSlots * kStagedColumns * w->shape.k * sizeof(uint16_t));
-    if (e != hipSuccess) return hip_fail(e, "hipMalloc(column staging)");
-    w->xrows_cols = kStagedColumns;
+    StreamSet &t = w->set[i];
+    if (!t.accum) {
+        const size_t bytes = set_words(w) * sizeof(unsigned long long);
+        hipError_t e = hipMalloc((void **)&t.accum, bytes);
+        if (e != hipSuccess) return hip_fail(e, "hipMalloc(split-k accumulators)");
+        e = hipMemset(t.accum, 0, bytes);
+        if (e != hipSuccess) return hip_fail(e, "hipMemset(split-k accumulators)");
+    }
+    if (!t.xrows) {
+        hipError_t e = hipMalloc(&t.xrows, (size_t)kStagedColumns * w->shape.k * sizeof(uint16_t));
+        if (e != hipSuccess) return hip_fail(e, "hipMalloc(column staging)");
+        t.xrows_cols = kStagedColumns;
+    }
     return LUTGEMM_OK;
 }
 
-// The split-k words launches on `stream` use.  The first launch of a stream on this handle claims
-// a set; kStreamSlots streams can use one handle at a time (clones have sets of their own).
-int stream_words(lutgemm_weight *w, void *stream, unsigned long long **words, int *slot)
+int alloc_workspace(lutgemm_weight *w)
+{
+    w->rows_per_set = batch_kernel_takes(w->shape) ? kRowsPerPass : kTableRows;
+    return alloc_set(w, 0);
+}
+
+size_t workspace_bytes(const lutgemm_weight *w)
+{
+    size_t bytes = 0;
+    for (int i = 0; i < kStreamSlots; i++) {
+        if (w->set[i].accum) bytes += set_words(w) * sizeof(unsigned long long);
+        if (w->set[i].xrows) bytes += (size_t)w->set[i].xrows_cols * w->shape.k * sizeof(uint16_t);
+    }
+    return bytes;
+}
+
+// The set launches on `stream` use.  The first launch of a stream on this handle claims one.
+int stream_set(lutgemm_weight *w, void *stream, int *slot)
 {
     std::lock_guard<std::mutex> lock(w->slot_mutex);
     for (int i = 0; i < w->slots_used; i++)
-        if (w->slot_stream[i] == stream) {
-            *words = w->d_accum + (size_t)i * w->slot_words;
+        if (w->set[i].stream == stream) {
+            w->set[i].last_use = ++w->use_clock;
             *slot = i;
             return LUTGEMM_OK;
         }
-    if (w->slots_used == kStreamSlots)
-        return fail(LUTGEMM_ERR_UNSUPPORTED,
-                    "more than %d streams have launched on this handle; use lutgemm_weight_clone for "
-                    "further streams or lutgemm_weight_reset_workspace to release the sets", kStreamSlots);
-    w->slot_stream[w->slots_used] = stream;
-    *words = w->d_accum + (size_t)w->slots_used * w->slot_words;
-    *slot = w->slots_used++;
+    int take = -1;
+    if (w->slots_used < kStreamSlots) {
+        take = w->slots_used;
+        if (int st = alloc_set(w, take)) return st;
+        if (!w->set[take].done) {
+            hipError_t e = hipEventCreateWithFlags(&w->set[take].done, hipEventDisableTiming);
+            if (e != hipSuccess) return hip_fail(e, "hipEventCreate");
+        }
+        w->slots_used++;
+    } else {
+        // all sets serve a stream: take over the least recently used one whose latest launch is known to
+        // have completed; failing that, the least recently used one with a recorded event, after making
+        // `stream` wait for it
+        int idle = -1, busy = -1;
+        for (int i = 0; i < kStreamSlots; i++) {
+            const StreamSet &t = w->set[i];
+            if (!t.done_valid) continue;
+            if (hipEventQuery(t.done) == hipSuccess) {
+                if (idle < 0 || t.last_use < w->set[idle].last_use) idle = i;
+            } else if (busy < 0 || t.last_use < w->set[busy].last_use) {
+                busy = i;
+            }
+        }
+        (void)hipGetLastError();  // hipErrorNotReady from the queries is not a failure
+        take = idle >= 0 ? idle : busy;
+        if (take < 0)
+            return fail(LUTGEMM_ERR_UNSUPPORTED,
+                        "%d streams use this handle and none of their sets can be taken over (launches under "
+                        "graph capture are not tracked); use lutgemm_weight_clone for further streams or "
+                        "lutgemm_weight_reset_workspace to release the sets", kStreamSlots);
+        if (idle < 0) {
+            hipError_t e = hipStreamWaitEvent(static_cast<hipStream_t>(stream), w->set[take].done, 0);
+            if (e != hipSuccess) return hip_fail(e, "hipStreamWaitEvent");
+        }
+    }
+    w->set[take].stream = stream;
+    w->set[take].done_valid = false;
+    w->set[take].last_use = ++w->use_clock;
+    *slot = take;
     return LUTGEMM_OK;
+}
+
+// Behind a launch on set `slot`: once the handle serves more than one stream, remember where the
+// stream stands, so that the set can be handed to another stream later.  A stream under capture
+// records nothing (the event would belong to the graph); its set is then not handed on.
+void note_launch(lutgemm_weight *w, int slot, void *stream)
+{
+    std::lock_guard<std::mutex> lock(w->slot_mutex);
+    if (w->slots_used < 2) return;
+    StreamSet &t = w->set[slot];
+    hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(static_cast<hipStream_t>(stream), &capturing) != hipSuccess ||
+        capturing != hipStreamCaptureStatusNone) {
+        (void)hipGetLastError();
+        t.done_valid = false;
+        return;
+    }
+    t.done_valid = hipEventRecord(t.done, static_cast<hipStream_t>(stream)) == hipSuccess;
 }
 
 // The allocation-free entry point marks a device whose static split-k words a failed call may
 // have left non-zero; the next call on that device clears them first.
-bool g_static_dirty[lutgemm_kernels::kMaxDevices];
+std::atomic<bool> g_static_dirty[lutgemm_kernels::kMaxDevices];
 
 // New handle for shape s on the current device from tiles already in the device layout
 // (host or device memory, `kind` says which).
@@ -378,7 +460,7 @@ int create_from_tiles(const Shape &s, const void *signs, const void *scales, hip
     return LUTGEMM_OK;
 }
 
-void fill_info(const Shape &s, size_t accum_bytes, lutgemm_weight_info_t *info)
+void fill_info(const Shape &s, size_t workspace, lutgemm_weight_info_t *info)
 {
     info->k = s.k;
     info->n = s.n;
@@ -389,7 +471,7 @@ void fill_info(const Shape &s, size_t accum_bytes, lutgemm_weight_info_t *info)
     info->sign_bytes = (size_t)s.k / 8 * s.q * s.n;
     info->scale_bytes = (size_t)s.num_groups * s.q * s.n * 2;
     info->offset_bytes = s.has_offset ? (size_t)s.num_groups * s.n * 2 : 0;
-    info->device_bytes = sign_bytes(s) + scale_bytes(s) + accum_bytes;
+    info->device_bytes = sign_bytes(s) + scale_bytes(s) + workspace;
 }
 
 int shape_or_fail(int k, int n, int q, int num_groups, bool has_offset, Shape *s)
@@ -527,29 +609,34 @@ int run_matvec(const lutgemm_weight *w, const void *x, void *y, int m, void *str
                         words / kRowsPerPass);
         hipError_t es = lutgemm_kernels::static_split_k_words(w->device, &a.accum);
         if (es != hipSuccess) return hip_fail(es, "hipGetSymbolAddress(static split-k words)");
-        if (g_static_dirty[w->device]) {  // a launch failed half way through a call: start from zero again
+        if (g_static_dirty[w->device].exchange(false)) {  // a launch failed half way through a call: start from zero again
             hipError_t e = lutgemm_kernels::launch_fill_zero(a.accum, words, st);
-            if (e != hipSuccess) return hip_fail(e, "launch fill_zero_kernel");
-            g_static_dirty[w->device] = false;
+            if (e != hipSuccess) {
+                g_static_dirty[w->device] = true;
+                return hip_fail(e, "launch fill_zero_kernel");
+            }
         }
-    } else if (int st_ws = stream_words(mw, stream, &a.accum, &slot)) {
-        return st_ws;
+    } else {
+        if (int st_ws = stream_set(mw, stream, &slot)) return st_ws;
+        a.accum = mw->set[slot].accum;
     }
     if (cols && m > 1) {
-        // gather the m columns into contiguous rows first (the kernel reads 16 bytes per lane)
-        if (m > mw->xrows_cols) {
-            // an earlier launch on any stream may still read the old buffer
+        // gather the m columns into contiguous rows first (the kernel reads 16 bytes per lane); the
+        // staging rows belong to the stream's set, or, for the allocation-free entry point, to set 0
+        StreamSet &t = mw->set[slot];
+        if (m > t.xrows_cols) {
+            // earlier launches of this stream may still read the old buffer
+            hipError_t e = hipStreamSynchronize(st);
+            if (e != hipSuccess) return hip_fail(e, "hipStreamSynchronize");
             std::lock_guard<std::mutex> lock(mw->slot_mutex);
-            hipError_t e = hipDeviceSynchronize();
-            if (e != hipSuccess) return hip_fail(e, "hipDeviceSynchronize");
-            if (mw->d_xrows) (void)hipFree(mw->d_xrows);
-            mw->d_xrows = nullptr;
-            mw->xrows_cols = 0;
-            e = hipMalloc(&mw->d_xrows, (size_t)kStreamSlots * m * s.k * sizeof(uint16_t));
+            if (t.xrows) (void)hipFree(t.xrows);
+            t.xrows = nullptr;
+            t.xrows_cols = 0;
+            e = hipMalloc(&t.xrows, (size_t)m * s.k * sizeof(uint16_t));
             if (e != hipSuccess) return hip_fail(e, "hipMalloc(column staging)");
-            mw->xrows_cols = m;
+            t.xrows_cols = m;
         }
-        uint16_t *rows = static_cast<uint16_t *>(mw->d_xrows) + (size_t)slot * mw->xrows_cols * s.k;
+        uint16_t *rows = static_cast<uint16_t *>(t.xrows);
         hipError_t e = lutgemm_kernels::launch_gather_columns(x, rows, s.k, m, st);
         if (e != hipSuccess) return hip_fail(e, "launch gather_columns_kernel");
         xh = rows;
@@ -582,6 +669,7 @@ int run_matvec(const lutgemm_weight *w, const void *x, void *y, int m, void *str
                 return hip_fail(e, "launch lut_batch_kernel");
             }
         }
+        if (!static_ws) note_launch(mw, slot, stream);
         return LUTGEMM_OK;
     }
     // two activation rows per pass over the weight, a last single row if m is odd
@@ -608,6 +696,7 @@ int run_matvec(const lutgemm_weight *w, const void *x, void *y, int m, void *str
             return hip_fail(e, "launch lut_matvec_kernel");
         }
     }
+    if (!static_ws) note_launch(mw, slot, stream);
     return LUTGEMM_OK;
 }
 
@@ -727,7 +816,12 @@ int lutgemm_weight_destroy(lutgemm_weight *w)
 {
     if (!w) return LUTGEMM_OK;
     int st = LUTGEMM_OK;
-    void *ptrs[4] = {w->d_signs, w->d_scales, w->d_accum, w->d_xrows};
+    std::vector<void *> ptrs = {w->d_signs, w->d_scales};
+    for (StreamSet &t : w->set) {
+        ptrs.push_back(t.accum);
+        ptrs.push_back(t.xrows);
+        if (t.done) (void)hipEventDestroy(t.done);
+    }
     for (void *p : ptrs)
         if (p) {
             hipError_t e = hipFree(p);
@@ -740,7 +834,7 @@ int lutgemm_weight_destroy(lutgemm_weight *w)
 int lutgemm_weight_info(const lutgemm_weight *w, lutgemm_weight_info_t *info)
 {
     if (!w || !info) return fail(LUTGEMM_ERR_NULL_POINTER, "null argument to weight_info");
-    fill_info(w->shape, w->accum_bytes, info);
+    fill_info(w->shape, workspace_bytes(w), info);
     return LUTGEMM_OK;
 }
 
@@ -761,9 +855,13 @@ int lutgemm_weight_reset_workspace(lutgemm_weight *w, void *stream)
     std::lock_guard<std::mutex> lock(w->slot_mutex);
     hipError_t e = hipDeviceSynchronize();  // no launch may still be using the words
     if (e != hipSuccess) return hip_fail(e, "hipDeviceSynchronize");
-    e = lutgemm_kernels::launch_fill_zero(w->d_accum, w->accum_bytes / sizeof(unsigned long long),
-                                          static_cast<hipStream_t>(stream));
-    if (e != hipSuccess) return hip_fail(e, "launch fill_zero_kernel");
+    for (StreamSet &t : w->set) {
+        t.stream = nullptr;
+        t.done_valid = false;
+        if (!t.accum) continue;
+        e = lutgemm_kernels::launch_fill_zero(t.accum, set_words(w), static_cast<hipStream_t>(stream));
+        if (e != hipSuccess) return hip_fail(e, "launch fill_zero_kernel");
+    }
     e = hipStreamSynchronize(static_cast<hipStream_t>(stream));
     if (e != hipSuccess) return hip_fail(e, "hipStreamSynchronize");
     w->slots_used = 0;
@@ -812,7 +910,7 @@ int lutgemm_matvec_many(const lutgemm_weight *const *ws, const void *const *xs, 
         lutgemm_kernels::MultiMatvecArgs multi{};
         Range xr[lutgemm_kernels::kMaxFused], yr[lutgemm_kernels::kMaxFused];
         const Shape *shapes[lutgemm_kernels::kMaxFused];
-        int rows_of[lutgemm_kernels::kMaxFused];
+        int rows_of[lutgemm_kernels::kMaxFused], slots[lutgemm_kernels::kMaxFused];
         int j = i;
         const lutgemm_weight *w0 = ws[i];
         const int kind = w0 && xs[i] && ys[i] ? kind_of(w0, ms[i]) : 0;
@@ -865,8 +963,9 @@ int lutgemm_matvec_many(const lutgemm_weight *const *ws, const void *const *xs, 
             a.k_splits = div_up(a.ts, a.blocks_per_split);
             multi.first_block[e] = blocks;
             blocks += a.ntiles * a.k_splits;
-            int slot = 0;
-            if (int st_ws = stream_words(const_cast<lutgemm_weight *>(ws[i + e]), stream, &a.accum, &slot)) return st_ws;
+            lutgemm_weight *we = const_cast<lutgemm_weight *>(ws[i + e]);
+            if (int st_ws = stream_set(we, stream, &slots[e])) return st_ws;
+            a.accum = we->set[slots[e]].accum;
         }
         multi.count = run;
         hipError_t e = kind != 2 ? lutgemm_kernels::launch_matvec_multi(w0->shape.q, w0->shape.has_offset, w0->shape.gsub, multi,
@@ -874,6 +973,7 @@ int lutgemm_matvec_many(const lutgemm_weight *const *ws, const void *const *xs, 
                                  : lutgemm_kernels::launch_batch_multi(w0->shape.q, w0->shape.has_offset, w0->shape.gsub, multi,
                                                                        blocks, fp.waves, static_cast<hipStream_t>(stream));
         if (e != hipSuccess) return hip_fail(e, kind != 2 ? "launch lut_matvec_multi_kernel" : "launch lut_batch_multi_kernel");
+        for (int en = 0; en < run; en++) note_launch(const_cast<lutgemm_weight *>(ws[i + en]), slots[en], stream);
         i = j;
     }
     return LUTGEMM_OK;

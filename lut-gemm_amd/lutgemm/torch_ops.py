@@ -6,7 +6,12 @@
 The operator launches on torch's current stream and allocates nothing but its output, so it can
 be captured into a HIP graph like any other torch op.  Batches larger than `dense_threshold`
 rows go through the dequantised fp16 weight and the library GEMM, the route the reference takes
-for every m > 1 (lutGEMM/src/kernels.cu:73-79); up to it the library streams the packed weight
+for every m > 1 (lutGEMM/src/kernels.cu:73-79).  Like the reference, which dequantises into one
+grow-only scratch buffer of the process on every such call (lutGEMM/src/cuda/tmpWeight.hpp:28-35,
+lutGEMM/src/nQWeight_fp16.cu:93-99), the dense weight is rebuilt per call in a scratch buffer shared
+by all layers (one per device and stream), so a layer never holds more than its packed weight;
+`keep_dense=True` keeps a private dense copy instead (2 k n bytes) and skips the rebuild.  Up to
+the threshold the library streams the packed weight
 (one or two rows through the table-lookup kernels, more through the batch kernel, 16 rows per
 pass).  The default threshold depends on the weight (default_dense_threshold): it is where the
 two routes met when measured on MI355X.
@@ -35,6 +40,18 @@ from . import BCQWeight, LutGemmError, ERR_BAD_SHAPE, MAX_BATCH
 
 _weights = weakref.WeakValueDictionary()  # operator argument (an int) -> BCQWeight
 _next_id = [1]
+_dense_scratch = {}   # (device index, stream handle) -> grow-only fp16 buffer for dequantised weights
+
+
+def dense_scratch(halves, device, stream_handle):
+    """View of `halves` fp16 elements of the process-wide scratch buffer of (device, stream); the
+    buffer only ever grows (the counterpart of the reference's tmpWeight singleton)."""
+    key = (device.index, stream_handle)
+    buf = _dense_scratch.get(key)
+    if buf is None or buf.numel() < halves:
+        buf = torch.empty(halves, dtype=torch.float16, device=device)
+        _dense_scratch[key] = buf
+    return buf[:halves]
 
 
 def register(weight):
@@ -82,9 +99,11 @@ class LutLinear(torch.nn.Module):
     container: dict(bW, alpha, q_bias, k, n, q, num_groups) as quantize.to_container returns.
     """
 
-    def __init__(self, container, bias=None, dense_threshold=None, autotune=False):
+    def __init__(self, container, bias=None, dense_threshold=None, autotune=False, keep_dense=False):
         super().__init__()
         c = container
+        self.device = torch.device("cuda", torch.cuda.current_device())   # the packed weight lives here
+        self.keep_dense = keep_dense
         self.weight = BCQWeight(c["bW"], c["alpha"], c["k"], c["n"], c["q"], c["num_groups"], c.get("q_bias"))
         if autotune:
             self.weight.autotune(torch.cuda.current_stream().cuda_stream)
@@ -93,7 +112,7 @@ class LutLinear(torch.nn.Module):
         self.dense_threshold = default_dense_threshold(self.weight) if dense_threshold is None else dense_threshold
         self._dense = None
         if bias is not None:
-            self.register_buffer("bias", torch.as_tensor(bias).to(torch.float16).cuda())
+            self.register_buffer("bias", torch.as_tensor(bias).to(torch.float16).to(self.device))
         else:
             self.bias = None
 
@@ -101,6 +120,8 @@ class LutLinear(torch.nn.Module):
     def from_file(cls, path, bias=None, **kw):
         self = cls.__new__(cls)
         torch.nn.Module.__init__(self)
+        self.device = torch.device("cuda", torch.cuda.current_device())
+        self.keep_dense = kw.get("keep_dense", False)
         self.weight = BCQWeight.load(path)
         if kw.get("autotune", False):
             self.weight.autotune(torch.cuda.current_stream().cuda_stream)
@@ -110,7 +131,7 @@ class LutLinear(torch.nn.Module):
         self.dense_threshold = default_dense_threshold(self.weight) if dt is None else dt
         self._dense = None
         if bias is not None:
-            self.register_buffer("bias", torch.as_tensor(bias).to(torch.float16).cuda())
+            self.register_buffer("bias", torch.as_tensor(bias).to(torch.float16).to(self.device))
         else:
             self.bias = None
         return self
@@ -124,13 +145,22 @@ class LutLinear(torch.nn.Module):
         return cls(c, bias=b, **kw)
 
     def dense_weight(self):
-        """Dequantised fp16 weight on the device as W^T [n][k] (built once, kept for large
-        batches): the orientation the dequantise kernel writes in 1 KiB runs."""
-        if self._dense is None:
-            Wt = torch.empty((self.out_features, self.in_features), dtype=torch.float16, device="cuda")
-            self.weight.dequantize(Wt.data_ptr(), True, torch.cuda.current_stream().cuda_stream)
+        """Dequantised fp16 weight on the layer's device as W^T [n][k], the orientation the
+        dequantise kernel writes in 1 KiB runs.  Rebuilt on torch's current stream into the shared
+        scratch buffer of that stream on every call (valid until the next layer's call on the
+        stream); with keep_dense it is built once and kept by the layer."""
+        if self._dense is not None:
+            return self._dense
+        stream = torch.cuda.current_stream(self.device).cuda_stream
+        if self.keep_dense:
+            Wt = torch.empty((self.out_features, self.in_features), dtype=torch.float16, device=self.device)
+        else:
+            Wt = dense_scratch(self.out_features * self.in_features, self.device, stream).view(self.out_features, self.in_features)
+        with torch.cuda.device(self.device):
+            self.weight.dequantize(Wt.data_ptr(), True, stream)
+        if self.keep_dense:
             self._dense = Wt
-        return self._dense
+        return Wt
 
     def forward(self, x):
         rows = x.numel() // x.shape[-1]

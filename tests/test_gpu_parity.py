@@ -695,6 +695,58 @@ def test_one_handle_on_two_streams(lutgemm, oracle, device):
     W.close()
 
 
+def test_one_handle_on_many_streams(lutgemm, oracle, device):
+    """A handle keeps four stream sets; further streams take over the set used least recently, waiting
+    for its launches if they have not completed: seven streams in sequence, then seven streams whose
+    launches overlap, then the column-batched form (staging rows per set), all bit-identical to the
+    same launches on one stream; the handle's memory grows by one set per further stream, up to four."""
+    import torch
+    from lutgemm import synth
+    k, n, q, g = 8192, 4096, 3, 128
+    w, W = make(lutgemm, synth, k, n, q, g, seed=18)
+    W.set_plan(8, 8)
+    xs = synth.make_x(7, k, seed=18)
+    xd = torch.from_numpy(xs).to(device)
+    serial = torch.zeros((7, n), dtype=torch.float16, device=device)
+    st = torch.cuda.current_stream().cuda_stream
+    one_set = W.info().device_bytes
+    for r in range(7):
+        W.matvec(xd[r].data_ptr(), serial[r].data_ptr(), 1, st)
+    torch.cuda.synchronize()
+    assert_within_tolerance(serial.cpu().numpy(), truth_of(oracle, w, xs), "serial")
+    assert W.info().device_bytes == one_set
+    streams = [torch.cuda.Stream() for _ in range(7)]
+    out = torch.zeros((7, n), dtype=torch.float16, device=device)
+    torch.cuda.synchronize()
+    say("case seven streams in sequence")
+    for r, s_ in enumerate(streams):
+        W.matvec(xd[r].data_ptr(), out[r].data_ptr(), 1, s_.cuda_stream)
+        s_.synchronize()
+    assert torch.equal(out, serial)
+    grown = W.info().device_bytes
+    assert grown > one_set and (grown - one_set) % 3 == 0, (one_set, grown)   # three further sets, no more
+    say("case seven streams overlapping")
+    many = torch.zeros((12, 7, n), dtype=torch.float16, device=device)
+    torch.cuda.synchronize()
+    for i in range(12):
+        for r, s_ in enumerate(streams):
+            W.matvec(xd[r].data_ptr(), many[i, r].data_ptr(), 1, s_.cuda_stream)
+    torch.cuda.synchronize()
+    assert torch.equal(many, serial.unsqueeze(0).expand_as(many))
+    assert W.info().device_bytes == grown
+    say("case column-batched form on seven streams")
+    xc = xd[:3].t().contiguous()                      # [k][3]
+    want = torch.zeros((n, 3), dtype=torch.float16, device=device)
+    W.matvec_cols(xc.data_ptr(), want.data_ptr(), 3, st)
+    torch.cuda.synchronize()
+    cols = torch.zeros((7, n, 3), dtype=torch.float16, device=device)
+    for r, s_ in enumerate(streams):
+        W.matvec_cols(xc.data_ptr(), cols[r].data_ptr(), 3, s_.cuda_stream)
+    torch.cuda.synchronize()
+    assert torch.equal(cols, want.unsqueeze(0).expand_as(cols))
+    W.close()
+
+
 def test_dense_gemv_comparator(lutgemm, device):
     """The plain streaming fp16 GEMV that the benchmark times next to the LUT kernel: fp32
     accumulation over fp16 inputs, rows whose length is not a multiple of the unrolled step, more

@@ -15,7 +15,10 @@ ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 CSRC = os.path.join(ROOT, "lut-gemm_amd", "csrc")
 
 
-def kernels_of(tmp_path, source):
+import pytest
+
+
+def kernels_of(tmp_path, source, kernel="lut_batch_kernel", args="10MatvecArgs"):
     out = os.path.join(str(tmp_path), "out.s")
     cmd = ["/opt/rocm/bin/hipcc", "-O3", "-std=c++17", "-fPIC", "--offload-arch=gfx950", "-Xclang", "-target-feature",
            "-Xclang", "-packed-fp32-ops", "-Wno-unused-command-line-argument", "-I", CSRC, "-S", "--cuda-device-only",
@@ -23,7 +26,7 @@ def kernels_of(tmp_path, source):
     subprocess.run(cmd, check=True, stdout=subprocess.DEVNULL, stderr=subprocess.DEVNULL)
     text = open(out).read()
     found = {}
-    for m in re.finditer(r"^(_ZN\S*lut_batch_kernel(\S*?)EEvNS_10MatvecArgsE):[^\n]*\n(.*?)s_endpgm", text, re.S | re.M):
+    for m in re.finditer(r"^(_ZN\S*%s(\S*?)EEvNS_%sE):[^\n]*\n(.*?)s_endpgm" % (kernel, args), text, re.S | re.M):
         body = [ln.strip() for ln in m.group(3).splitlines() if ln.strip() and not ln.strip().startswith(";")]
         meta = text[text.index(".amdhsa_kernel " + m.group(1)):]
         found[m.group(2)] = (body, meta[:meta.index(".end_amdhsa_kernel")])
@@ -47,6 +50,7 @@ def uses_of_registers_in_flight(body):
     and branches, which only makes the check stricter) and returns the instructions that read or
     write a VGPR while an LDS read into it is queued."""
     queue, bad = [], []
+    scalar_loads = False   # scalar memory loads count on the same counter and return in any order
     for line in body:
         line = line.split(";")[0].strip()
         if not line or line.endswith(":") or line.startswith("."):
@@ -57,7 +61,14 @@ def uses_of_registers_in_flight(body):
             m = re.search(r"lgkmcnt\((\d+)\)", rest)
             if m:
                 n = int(m.group(1))
+                if n > 0 and scalar_loads and any(queue):
+                    bad.append(line + "   ; partial wait for LDS reads with a scalar load outstanding")
+                if n == 0:
+                    scalar_loads = False
                 queue = queue[len(queue) - n:] if 0 < n < len(queue) else ([] if n == 0 else queue)
+            continue
+        if op.startswith(("s_load_", "s_buffer_load_")):
+            scalar_loads = True
             continue
         pending = set().union(*queue) if queue else set()
         if op.startswith("ds_"):
@@ -78,10 +89,22 @@ def test_the_in_flight_check_sees_a_short_wait():
     assert uses_of_registers_in_flight(good) == []
     assert uses_of_registers_in_flight([good[0], good[1], "s_waitcnt lgkmcnt(1)", "v_mov_b32_e32 v8, v5"]) == ["v_mov_b32_e32 v8, v5"]
     assert uses_of_registers_in_flight([good[0], "ds_write_b32 v9, v2"]) == ["ds_write_b32 v9, v2"]
+    # a scalar load shares the counter and may return after the LDS reads: a partial wait proves nothing
+    mixed = ["s_load_dwordx2 s[0:1], s[4:5], 0x0", good[0], good[1], "s_waitcnt lgkmcnt(1)", "v_mov_b32_e32 v8, v0"]
+    assert len(uses_of_registers_in_flight(mixed)) == 1
+    assert uses_of_registers_in_flight([mixed[0], "s_waitcnt lgkmcnt(0)"] + good) == []
 
 
-def test_batch_kernel_assembly(tmp_path):
-    kernels = kernels_of(tmp_path, "batch.hip")
+# register spills (scratch memory per lane, bytes) the instantiations may carry: none for two planes
+# without offset, the headline of the decoder-layer chain; the largest ones are the offset variants
+# with four scale groups per 128 k
+MAX_SCRATCH_BYTES = 128
+
+
+@pytest.mark.parametrize("source,kernel,args", [("batch.hip", "lut_batch_kernel", "10MatvecArgs"),
+                                                ("batch_multi.hip", "lut_batch_multi_kernel", "15MultiMatvecArgs")])
+def test_batch_kernel_assembly(tmp_path, source, kernel, args):
+    kernels = kernels_of(tmp_path, source, kernel, args)
     assert len(kernels) == 48, sorted(kernels)   # 4 plane counts x offset x 3 scale layouts x second staged row
     for name, (body, meta) in sorted(kernels.items()):
         ops = [ln.split()[0] for ln in body]
@@ -107,6 +130,8 @@ def test_batch_kernel_assembly(tmp_path):
         assert waits_before and "vmcnt(0)" in waits_before[-1], (name, waits_before)
         between = tail[stores[0]:stores[7]]   # (the stores of the path without k-splits follow behind a branch of their own)
         assert not [ln for ln in between if ln.startswith("s_waitcnt") and "vmcnt" in ln], name
+        scratch = int(re.search(r"\.amdhsa_private_segment_fixed_size (\d+)", meta).group(1))
+        assert scratch <= MAX_SCRATCH_BYTES, (name, scratch)
     # the headline instantiation of the decoder-layer chain (two planes, no offset, one group per 128 k): no scratch memory
     body, meta = kernels["ILi2ELb0ELi1ELi16ELb0E"]
     assert re.search(r"\.amdhsa_private_segment_fixed_size 0\b", meta)

@@ -44,7 +44,21 @@ def test_large_batches_take_the_dense_route(lutgemm, oracle, device):
     layer = torch_ops.LutLinear(c, dense_threshold=8)
     x = torch.randn(40, 1024, generator=gen).to(torch.float16)
     y_dense = layer(x.to(device))                       # 40 rows > threshold: dequantise + GEMM
-    assert layer._dense is not None and layer._dense.shape == (320, 1024)   # W^T [n][k]
+    # by default the layer keeps no dense copy: the weight is rebuilt per call in the scratch buffer
+    # all layers of the stream share, which only grows (what the reference's scratch singleton does)
+    assert layer._dense is None
+    scratch = torch_ops.dense_scratch(320 * 1024, layer.device, torch.cuda.current_stream().cuda_stream)
+    torch.cuda.synchronize()
+    shared = scratch.view(320, 1024).clone()            # W^T [n][k]
+    small = torch_ops.LutLinear(quantize.quantize_linear(lin.weight.detach()[:64], 4, 128, "rtn")[0], dense_threshold=8)
+    y_small = small(x.to(device))
+    assert torch_ops.dense_scratch(1, layer.device, torch.cuda.current_stream().cuda_stream).data_ptr() == scratch.data_ptr()
+    assert torch.allclose(y_small.float(), y_dense[:, :64].float(), atol=2e-2, rtol=0)   # another GEMM shape
+    assert torch.equal(layer(x.to(device)), y_dense)     # rebuilt after another layer used the scratch
+    kept = torch_ops.LutLinear(c, dense_threshold=8, keep_dense=True)
+    assert torch.equal(kept(x.to(device)), y_dense)
+    assert kept._dense is not None and kept._dense.shape == (320, 1024) and torch.equal(kept._dense, shared)
+    layer._dense = shared                               # for the checks below
     y_lut = torch.ops.lutgemm.matvec(x.to(device), layer.handle)
     # the dense weight is the oracle's dense weight rounded to fp16
     a16 = c["alpha"].astype(np.float16)
