@@ -92,8 +92,8 @@ int lutgemm_weight_info(const lutgemm_weight *w, lutgemm_weight_info_t *info);
  * 1 <= m <= LUTGEMM_MAX_BATCH streams the packed weight: m == 1 and m == 2 through the table-lookup
  * kernels (a two-row pass gives each row bit-identical to its own one-row call), m >= 3 through
  * the batch kernel, which takes up to 16 rows per pass over the weight and contracts them on the
- * matrix cores while a tile is in registers (weights of up to four planes, any group size; weights
- * of more planes take table-lookup passes of two rows).  Batch results are deterministic and within
+ * matrix cores while a tile is in registers (any number of planes and any group size; weights of
+ * more than four planes with workgroups of exactly eight wavefronts).  Batch results are deterministic and within
  * the same tolerance, but a row may differ in the last bit from its own one-row call (another order
  * of the fp32 additions).
  * Launches on one stream run one after the other and share one set of split-k accumulators of the
@@ -139,7 +139,7 @@ int lutgemm_matvec_cols(const lutgemm_weight *w, const void *x, void *y, int m, 
  * computes ys[i] = xs[i] * ws[i] with batch ms[i] exactly as lutgemm_matvec would, and the results
  * are those of the entries executed in order.  Consecutive entries that do not depend on each other
  * share ONE kernel launch (up to 32 per launch): entries that all have one activation row, that all
- * have two, or that all have 3 to 16 rows on weights of up to four planes (the batch kernel), with the same q /
+ * have two, or that all have 3 to 16 rows (the batch kernel), with the same q /
  * offset / group layout, distinct handles, and no output overlapping an input or output of another
  * entry of the launch.  The workgroups of such entries follow each other in one grid, so the memory
  * system stays busy while single workgroups start and finish, and the launch overhead is paid
@@ -147,10 +147,35 @@ int lutgemm_matvec_cols(const lutgemm_weight *w, const void *x, void *y, int m, 
  * the whole run, not the handles' plans, so a result may differ in the last bit from the same
  * entry's lutgemm_matvec call; it is deterministic (same entries, same bits) and within the same
  * tolerance.  Entries that do not qualify (a later entry reading an earlier output, more than 16
- * rows, three and more rows on more than four planes, another kernel instance) get launches of their own, in order, exactly as lutgemm_matvec issues them.  Has no counterpart in the reference, whose caller loops over lutGEMM::matmul
+ * rows, another kernel instance) get launches of their own, in order, exactly as lutgemm_matvec issues them.  Has no counterpart in the reference, whose caller loops over lutGEMM::matmul
  * itself (tests/opt/fp16/int3_col_wise_matmul_fp16.cu:120-133).  Stops at the first failing entry. */
 int lutgemm_matvec_many(const lutgemm_weight *const *ws, const void *const *xs, void *const *ys,
                         const int *ms, int count, void *stream);
+
+/* Replace the model's choice of the launch shape of fused launches by a measurement.  Walks the
+ * list as lutgemm_matvec_many does; for every run of entries that share a launch it times the six
+ * launch shapes (wavefronts per workgroup, k-blocks per workgroup) the cost model ranks best, the
+ * model's own choice among them, with the entries themselves on `stream` (a few launches each; ys
+ * receive valid results; the device is kept busy for 30 ms first so that the clocks are up) and
+ * remembers the fastest, process-wide, under the shapes of the run: kernel instance, compute units,
+ * and (k, n, rows) of its entries in order.  From then on every lutgemm_matvec_many run of those
+ * shapes, whatever its handles and buffers, is launched that way.  The constants of the cost model
+ * were fitted on one MI355X; this call is how a caller checks them on the box it runs on.
+ * The buffers are measured as they are: a list whose weights fit the memory-side cache is timed
+ * from that cache.  Entries that do not share a launch are launched once, as lutgemm_matvec does
+ * (their plans belong to the handles: lutgemm_weight_autotune).  Synchronises `stream`.  No
+ * counterpart in the reference, whose tile sizes are fixed
+ * (lutGEMM/src/cuda/kernels/mv_fp16.hpp:122-124). */
+int lutgemm_matvec_many_autotune(const lutgemm_weight *const *ws, const void *const *xs, void *const *ys,
+                                 const int *ms, int count, void *stream);
+
+/* The launch shape lutgemm_matvec_many would use for the first launch of this list, for tests and
+ * benchmarks: how many entries share it (1: the first entry is launched on its own and the other
+ * outputs are 0), wavefronts and k-blocks per workgroup, and whether that shape was measured by
+ * lutgemm_matvec_many_autotune (1) or comes from the cost model (0).  Any output may be NULL. */
+int lutgemm_matvec_many_plan(const lutgemm_weight *const *ws, const void *const *xs, void *const *ys,
+                             const int *ms, int count, int *entries_in_first_launch, int *waves_per_group,
+                             int *k_blocks_per_group, int *measured);
 
 /* As lutgemm_matvec_many, but every entry gets a launch of its own (the call is a plain loop over
  * lutgemm_matvec): for per-launch timing and profiling. */
@@ -200,8 +225,7 @@ int lutgemm_weight_plan(const lutgemm_weight *w, int *workgroups, int *waves_per
                         int *k_splits, int *k_blocks_per_group);
 
 /* The same for the launches a call with m activation rows makes (m = 1: the plan above; m = 2:
- * the two-row plan; m >= 3: the batch kernel's plan for passes of min(m, 16) rows where the
- * weight has up to four planes, else the two-row plan).  LUTGEMM_ERR_BAD_SHAPE for m outside
+ * the two-row plan; m >= 3: the batch kernel's plan for passes of min(m, 16) rows).  LUTGEMM_ERR_BAD_SHAPE for m outside
  * 1..LUTGEMM_MAX_BATCH.  No counterpart in the reference. */
 int lutgemm_weight_plan_for(const lutgemm_weight *w, int m, int *workgroups, int *waves_per_group,
                             int *k_splits, int *k_blocks_per_group);
@@ -212,10 +236,11 @@ int lutgemm_weight_plan_for(const lutgemm_weight *w, int m, int *workgroups, int
  * (1..12 wavefronts per workgroup, 1..min(k/512 rounded up, 128) k-splits). */
 int lutgemm_weight_set_plan(lutgemm_weight *w, int waves_per_group, int k_splits);
 
-/* Override the batch kernel's launch plan (calls with 3 or more rows on weights of up to four
- * planes): 8..16 wavefronts per workgroup and the k-splits; both 0: back to the automatic choice.
- * LUTGEMM_ERR_BAD_SHAPE if the request cannot be launched, LUTGEMM_ERR_UNSUPPORTED for weights
- * that never take the batch kernel.  No launch on the handle may be in flight. */
+/* Override the batch kernel's launch plan (calls with 3 or more rows): 8..16 wavefronts per
+ * workgroup (exactly 8 for weights of more than four planes; fewer than 16 where four scale
+ * groups per 128 k leave less LDS) and the k-splits; both 0: back to the automatic choice.
+ * LUTGEMM_ERR_BAD_SHAPE if the request cannot be launched.  No launch on the handle may be in
+ * flight. */
 int lutgemm_weight_set_batch_plan(lutgemm_weight *w, int waves_per_group, int k_splits);
 
 /* Measure the most promising launch plans on the device (a few launches each, on `stream`, with

@@ -554,19 +554,29 @@ __device__ __forceinline__ void batch_workgroup(const MatvecArgs &a, unsigned bl
 }
 
 
-// Launches kernel<Q, OFF, GSUB, kBatchWaves, TWO>(args) for the runtime (q, has_offset, gsub, rows
-// against wavefronts): the same dispatch for the kernel of one batch and for the work-list kernel.
+// Launches kernel<Q, OFF, GSUB, W, TWO>(args) for the runtime (q, has_offset, gsub, rows against
+// wavefronts): the same dispatch for the kernel of one batch and for the work-list kernel.  W, the
+// largest workgroup the kernel is compiled for, is kBatchWaves for up to kBatchWidePlanes planes and
+// kBatchWavesMin beyond (one instantiation there, the one that stages two rows per wavefront: it
+// serves every batch size).
 // Launcher<Q, OFF, GSUB, W, TWO>::run(args, workgroups, waves, stream) is provided by the includer.
 template <template <int, bool, int, int, bool> class Launcher, typename Args>
 hipError_t dispatch_batch(int q, int has_offset, int gsub, bool two, const Args &args, int workgroups, int waves,
                           hipStream_t stream)
 {
-    constexpr int W = kBatchWaves;
     if (gsub != 1 && gsub != 2 && gsub != 4) return hipErrorInvalidValue;
     auto by_gsub = [&](auto Qc, auto OFFc) -> hipError_t {
         constexpr int Q = decltype(Qc)::value;
         constexpr bool OFF = decltype(OFFc)::value;
-        if (waves < kBatchWavesMin || waves > batch_waves_max(gsub, Q + (OFF ? 1 : 0))) return hipErrorInvalidValue;
+        constexpr int W = Q > kBatchWidePlanes ? kBatchWavesMin : kBatchWaves;
+        if (waves < kBatchWavesMin || waves > batch_waves_max(gsub, Q, Q + (OFF ? 1 : 0))) return hipErrorInvalidValue;
+        if constexpr (Q > kBatchWidePlanes) {
+            switch (gsub) {
+                case 1: return Launcher<Q, OFF, 1, W, true>::run(args, workgroups, waves, stream);
+                case 2: return Launcher<Q, OFF, 2, W, true>::run(args, workgroups, waves, stream);
+                default: return Launcher<Q, OFF, 4, W, true>::run(args, workgroups, waves, stream);
+            }
+        } else
         switch (gsub) {
             case 1: return two ? Launcher<Q, OFF, 1, W, true>::run(args, workgroups, waves, stream)
                                : Launcher<Q, OFF, 1, W, false>::run(args, workgroups, waves, stream);
@@ -584,6 +594,10 @@ hipError_t dispatch_batch(int q, int has_offset, int gsub, bool two, const Args 
         case 2: return by_offset(std::integral_constant<int, 2>{});
         case 3: return by_offset(std::integral_constant<int, 3>{});
         case 4: return by_offset(std::integral_constant<int, 4>{});
+        case 5: return by_offset(std::integral_constant<int, 5>{});
+        case 6: return by_offset(std::integral_constant<int, 6>{});
+        case 7: return by_offset(std::integral_constant<int, 7>{});
+        case 8: return by_offset(std::integral_constant<int, 8>{});
         default: return hipErrorInvalidValue;   // more planes than kBatchMaxPlanes
     }
 }
@@ -599,7 +613,7 @@ hipError_t allow_batch_lds(Kernel kernel, std::atomic<unsigned long long> &allow
     const unsigned long long bit = 1ull << (dev & 63);
     if (!(allowed.load(std::memory_order_relaxed) & bit)) {
         e = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                batch_lds_bytes(batch_waves_max(GSUB, QO), GSUB, QO));
+                                batch_lds_bytes(batch_waves_max(GSUB, Q, QO), GSUB, QO));
         if (e != hipSuccess) return e;
         allowed.fetch_or(bit, std::memory_order_relaxed);
     }

@@ -12,6 +12,7 @@
 #include <cstdint>
 #include <cstdio>
 #include <cstring>
+#include <map>
 #include <mutex>
 #include <new>
 #include <vector>
@@ -67,7 +68,7 @@ struct Plan {
 // launch records the set's event once the handle serves more than one stream.
 struct StreamSet {
     void *stream;                // the stream the set serves
-    unsigned long long *accum;   // rows_per_set x (padded outputs) split-k words, zero between launches
+    unsigned long long *accum;   // kRowsPerPass x (padded outputs) split-k words, zero between launches
     void *xrows;                 // staging of column-batched activations: xrows_cols rows of k halves,
     int xrows_cols;              //   grown on demand
     hipEvent_t done;             // recorded behind the set's latest launch (only while done_valid)
@@ -81,7 +82,6 @@ struct lutgemm_weight {
     int compute_units;
     uint8_t *d_signs;
     uint16_t *d_scales;
-    int rows_per_set;             // activation rows a launch on this weight can take: 16 (batch kernel) or 2
     std::mutex slot_mutex;
     StreamSet set[kStreamSlots];
     int slots_used;               // sets that serve a stream
@@ -157,7 +157,11 @@ Plan choose_plan(const Shape &s, int cus)
 // to measured times of 40 plans over five weight shapes and run lengths 3 to 32 on MI355X.
 struct FusedPlan { int waves, blocks_per_group; };
 
-FusedPlan choose_fused_plan(const Shape *const *shapes, int count, int cus, int rows)
+struct FusedCandidate { double cost; FusedPlan plan; };
+
+// `all` (optional) receives every launch shape the model considered with its cost
+FusedPlan choose_fused_plan(const Shape *const *shapes, int count, int cus, int rows,
+                            std::vector<FusedCandidate> *all = nullptr)
 {
     // two-row passes: a k-block builds and looks up two table sets, bound by the lookups
     const double kBytesPerCu = (rows == 2 ? 4.8e6 : 7.0e6) / 256.0;  // streaming rate per compute unit with all units busy
@@ -186,6 +190,7 @@ FusedPlan choose_fused_plan(const Shape *const *shapes, int count, int cus, int 
             const long full = groups / cus, rest = groups % cus;
             double cost = (double)full * (per_group + start_end);
             if (rest) cost += per_group * std::pow((double)rest / cus, kPartialExponent) + start_end;
+            if (all) all->push_back(FusedCandidate{cost, FusedPlan{waves, bpg}});
             if (cost < best_cost - 1e-9) {
                 best_cost = cost;
                 best = FusedPlan{waves, bpg};
@@ -219,7 +224,7 @@ double batch_plan_cost(const Shape &s, int cus, int waves, int ks, int rows, Pla
 // `rows`: 8 for passes of up to 8 rows, 16 for larger ones (the two plans a handle keeps)
 Plan choose_batch_plan(const Shape &s, int cus, int rows)
 {
-    const int wmax = lutgemm_kernels::batch_waves_max(s.gsub, s.qo), wmin = lutgemm_kernels::kBatchWavesMin;
+    const int wmax = lutgemm_kernels::batch_waves_max(s.gsub, s.q, s.qo), wmin = lutgemm_kernels::kBatchWavesMin;
     Plan best{wmax, div_up(s.nb, wmax), s.ts, 1};
     double best_cost = 1e30;
     for (int waves = wmin; waves <= wmax; waves++)
@@ -234,10 +239,7 @@ Plan choose_batch_plan(const Shape &s, int cus, int rows)
     return best;
 }
 
-bool batch_kernel_takes(const Shape &s)
-{
-    return s.q <= lutgemm_kernels::kBatchMaxPlanes;
-}
+static_assert(lutgemm_kernels::kBatchMaxPlanes == 8, "the batch kernel takes every plane count a weight can have");
 
 // Launch shape of several independent batches in one grid (lutgemm_matvec_many): one number of
 // wavefronts per workgroup and one number of k-blocks per workgroup for all entries.  The grid
@@ -248,14 +250,15 @@ bool batch_kernel_takes(const Shape &s)
 // the memory side executes them at a fixed rate.  Constants (microseconds) fitted to measured
 // times of 330 plans over eight lists (3 to 12 entries, k and n 2048 to 12288, 1 to 4 planes,
 // 4 to 16 rows) on MI355X; the fit names the fastest measured plan of each list.
-FusedPlan choose_fused_batch_plan(const Shape *const *shapes, const int *rows, int count, int cus)
+FusedPlan choose_fused_batch_plan(const Shape *const *shapes, const int *rows, int count, int cus,
+                                  std::vector<FusedCandidate> *all = nullptr)
 {
     const double tile_us = 0.110, two_rows = 1.165, block_us = 0.35, group_us = 3.0, group_wave_us = 0.30;
     const double atomic_us = 2.5e-6;
     int max_ts = 1, wmax = lutgemm_kernels::kBatchWaves;
     for (int e = 0; e < count; e++) {
         max_ts = shapes[e]->ts > max_ts ? shapes[e]->ts : max_ts;
-        const int w = lutgemm_kernels::batch_waves_max(shapes[e]->gsub, shapes[e]->qo);
+        const int w = lutgemm_kernels::batch_waves_max(shapes[e]->gsub, shapes[e]->q, shapes[e]->qo);
         wmax = w < wmax ? w : wmax;
     }
     FusedPlan best{wmax, max_ts};
@@ -278,6 +281,7 @@ FusedPlan choose_fused_batch_plan(const Shape *const *shapes, const int *rows, i
             const double per_group = work / (double)groups;
             const long rounds = (groups + cus - 1) / cus;
             const double cost = (double)rounds * per_group + atomic_us * atomics;
+            if (all) all->push_back(FusedCandidate{cost, FusedPlan{waves, bpg}});
             if (cost < best_cost - 1e-9) {
                 best_cost = cost;
                 best = FusedPlan{waves, bpg};
@@ -297,7 +301,7 @@ int check_device(const lutgemm_weight *w)
     return LUTGEMM_OK;
 }
 
-size_t set_words(const lutgemm_weight *w) { return (size_t)w->rows_per_set * w->shape.nb * kBatch; }
+size_t set_words(const lutgemm_weight *w) { return (size_t)kRowsPerPass * w->shape.nb * kBatch; }
 
 // Device memory of set i (idempotent).  Allocates: not for a stream that is being captured.
 int alloc_set(lutgemm_weight *w, int i)
@@ -320,7 +324,6 @@ int alloc_set(lutgemm_weight *w, int i)
 
 int alloc_workspace(lutgemm_weight *w)
 {
-    w->rows_per_set = batch_kernel_takes(w->shape) ? kRowsPerPass : kTableRows;
     return alloc_set(w, 0);
 }
 
@@ -643,7 +646,7 @@ int run_matvec(const lutgemm_weight *w, const void *x, void *y, int m, void *str
     }
     a.x_row_stride = s.k;
     a.accum_row_stride = (long long)s.nb * kBatch;
-    if (m >= 3 && batch_kernel_takes(s)) {
+    if (m >= 3) {
         // up to 16 rows per pass over the weight on the matrix cores
         const int pass_rows = m < kRowsPerPass ? m : kRowsPerPass;
         const Plan plan = w->batch_measured[pass_rows > 8] ? w->plan_batch[pass_rows > 8]
@@ -697,6 +700,156 @@ int run_matvec(const lutgemm_weight *w, const void *x, void *y, int m, void *str
         }
     }
     if (!static_ws) note_launch(mw, slot, stream);
+    return LUTGEMM_OK;
+}
+
+// ---- runs of independent entries that share one launch (lutgemm_matvec_many) ----------------
+// kind: 1 one-row entries, 3 two-row entries (table-lookup kernels), 2 batches of 3 to 16 rows (the
+// batch kernel); an entry of more than 16 rows is launched on its own.
+struct FusedRun {
+    int kind, count;
+    lutgemm_kernels::MultiMatvecArgs multi;
+    const lutgemm_weight *handle[lutgemm_kernels::kMaxFused];
+    const Shape *shape[lutgemm_kernels::kMaxFused];
+    int rows[lutgemm_kernels::kMaxFused];
+};
+
+int fused_kind(int m)
+{
+    if (m == 1) return 1;
+    if (m == 2) return 3;
+    if (m >= 3 && m <= kRowsPerPass) return 2;
+    return 0;
+}
+
+// Longest run of entries starting at i that one launch can take: the same kind and kernel
+// instance, no handle twice (its split-k words would be shared), and no output overlapping an
+// input or output of another entry of the run, so that their order does not matter.  Returns the
+// index behind the run (run->count is 0 when entry i cannot share a launch at all).
+int form_run(const lutgemm_weight *const *ws, const void *const *xs, void *const *ys, const int *ms, int count, int i,
+             FusedRun *run)
+{
+    struct Range { uintptr_t lo, hi; };
+    auto overlap = [](const Range &a, const Range &b) { return a.lo < b.hi && b.lo < a.hi; };
+    Range xr[lutgemm_kernels::kMaxFused], yr[lutgemm_kernels::kMaxFused];
+    run->multi = lutgemm_kernels::MultiMatvecArgs{};
+    int j = i;
+    const lutgemm_weight *w0 = ws[i];
+    const int kind = w0 && xs[i] && ys[i] ? fused_kind(ms[i]) : 0;
+    for (; kind != 0 && j < count && j - i < lutgemm_kernels::kMaxFused; j++) {
+        const lutgemm_weight *w = ws[j];
+        if (!w || !xs[j] || !ys[j] || ((uintptr_t)xs[j] & 15u) != 0 || fused_kind(ms[j]) != kind) break;
+        const Shape &s = w->shape;
+        if (s.q != w0->shape.q || s.has_offset != w0->shape.has_offset || s.gsub != w0->shape.gsub ||
+            w->device != w0->device)
+            break;
+        const int e = j - i;
+        xr[e] = Range{(uintptr_t)xs[j], (uintptr_t)xs[j] + (size_t)ms[j] * s.k * 2};
+        yr[e] = Range{(uintptr_t)ys[j], (uintptr_t)ys[j] + (size_t)ms[j] * s.n * 2};
+        bool independent = true;
+        for (int p = 0; p < e && independent; p++)
+            independent = ws[i + p] != w && !overlap(yr[e], yr[p]) && !overlap(yr[e], xr[p]) && !overlap(xr[e], yr[p]);
+        if (!independent) break;
+        run->handle[e] = w;
+        run->shape[e] = &s;
+        run->rows[e] = ms[j];
+        lutgemm_kernels::MatvecArgs &a = run->multi.entry[e];
+        a.signs = w->d_signs;
+        a.scales = w->d_scales;
+        a.k = s.k;
+        a.n = s.n;
+        a.ts = s.ts;
+        a.nb = s.nb;
+        a.x = xs[j];
+        a.y = ys[j];
+        a.y_stride = 1;
+        a.rows = ms[j];
+        a.x_row_stride = s.k;
+        a.y_row_stride = s.n;
+        a.accum_row_stride = (long long)s.nb * kBatch;
+    }
+    run->kind = kind;
+    run->count = j - i;
+    return j;
+}
+
+FusedPlan model_fused_plan(const FusedRun &run, std::vector<FusedCandidate> *all)
+{
+    const int cus = run.handle[0]->compute_units;
+    return run.kind == 2 ? choose_fused_batch_plan(run.shape, run.rows, run.count, cus, all)
+                         : choose_fused_plan(run.shape, run.count, cus, run.kind == 1 ? 1 : 2, all);
+}
+
+// two plans that give every entry of the run the same grid
+bool same_launch(const FusedRun &run, const FusedPlan &a, const FusedPlan &b)
+{
+    if (a.waves != b.waves) return false;
+    for (int e = 0; e < run.count; e++) {
+        const int ts = run.shape[e]->ts;
+        if ((a.blocks_per_group < ts ? a.blocks_per_group : ts) != (b.blocks_per_group < ts ? b.blocks_per_group : ts)) return false;
+    }
+    return true;
+}
+
+// Launch shapes measured by lutgemm_matvec_many_autotune, by what a run looks like: kind, kernel
+// instance, compute units and the (k, n, rows) of its entries in order.  Any list with the same
+// shapes finds the plan again, whatever its handles and buffers.
+constexpr size_t kFusedCandidates = 6;
+std::mutex g_fused_mutex;
+std::map<std::vector<int>, FusedPlan> g_fused_plans;
+
+std::vector<int> fused_key(const FusedRun &run)
+{
+    const Shape &s0 = *run.shape[0];
+    std::vector<int> key = {run.kind, s0.q, s0.has_offset, s0.gsub, run.handle[0]->compute_units, run.count};
+    for (int e = 0; e < run.count; e++) {
+        key.push_back(run.shape[e]->k);
+        key.push_back(run.shape[e]->n);
+        key.push_back(run.rows[e]);
+    }
+    return key;
+}
+
+bool measured_fused_plan(const FusedRun &run, FusedPlan *out)
+{
+    std::lock_guard<std::mutex> lock(g_fused_mutex);
+    if (g_fused_plans.empty()) return false;
+    const auto it = g_fused_plans.find(fused_key(run));
+    if (it == g_fused_plans.end()) return false;
+    *out = it->second;
+    return true;
+}
+
+void remember_fused_plan(const FusedRun &run, const FusedPlan &plan)
+{
+    std::lock_guard<std::mutex> lock(g_fused_mutex);
+    g_fused_plans[fused_key(run)] = plan;
+}
+
+// One launch for the run with launch shape fp (asynchronous).
+int launch_run(FusedRun &run, const FusedPlan &fp, void *stream)
+{
+    const Shape &s0 = *run.shape[0];
+    int slots[lutgemm_kernels::kMaxFused];
+    int blocks = 0;
+    for (int e = 0; e < run.count; e++) {
+        lutgemm_kernels::MatvecArgs &a = run.multi.entry[e];
+        a.ntiles = div_up(a.nb, fp.waves);
+        a.blocks_per_split = fp.blocks_per_group < a.ts ? fp.blocks_per_group : a.ts;
+        a.k_splits = div_up(a.ts, a.blocks_per_split);
+        run.multi.first_block[e] = blocks;
+        blocks += a.ntiles * a.k_splits;
+        lutgemm_weight *we = const_cast<lutgemm_weight *>(run.handle[e]);
+        if (int st_ws = stream_set(we, stream, &slots[e])) return st_ws;
+        a.accum = we->set[slots[e]].accum;
+    }
+    run.multi.count = run.count;
+    hipError_t e = run.kind != 2 ? lutgemm_kernels::launch_matvec_multi(s0.q, s0.has_offset, s0.gsub, run.multi, blocks, fp.waves,
+                                                                       static_cast<hipStream_t>(stream))
+                                 : lutgemm_kernels::launch_batch_multi(s0.q, s0.has_offset, s0.gsub, run.multi, blocks, fp.waves,
+                                                                       static_cast<hipStream_t>(stream));
+    if (e != hipSuccess) return hip_fail(e, run.kind != 2 ? "launch lut_matvec_multi_kernel" : "launch lut_batch_multi_kernel");
+    for (int en = 0; en < run.count; en++) note_launch(const_cast<lutgemm_weight *>(run.handle[en]), slots[en], stream);
     return LUTGEMM_OK;
 }
 
@@ -890,92 +1043,117 @@ int lutgemm_matvec_many(const lutgemm_weight *const *ws, const void *const *xs, 
 {
     if (!ws || !xs || !ys || !ms) return fail(LUTGEMM_ERR_NULL_POINTER, "null argument to matvec_many");
     if (count < 0) return fail(LUTGEMM_ERR_BAD_SHAPE, "count=%d is negative", count);
-    struct Range { uintptr_t lo, hi; };
-    auto overlap = [](const Range &a, const Range &b) { return a.lo < b.hi && b.lo < a.hi; };
-    // what one launch can take: one-row entries or two-row entries (table-lookup kernels), or batches
-    // of 3 to 16 rows of weights the batch kernel takes; anything else (more than 16 rows, more than
-    // four planes with three rows and up) is launched on its own
-    auto kind_of = [](const lutgemm_weight *w, int m) {
-        if (m == 1) return 1;
-        if (m == 2) return 3;
-        if (m >= 3 && m <= kRowsPerPass && batch_kernel_takes(w->shape)) return 2;
-        return 0;
-    };
     int i = 0;
     while (i < count) {
-        // Longest run of entries starting at i that one launch can take: the same kind and kernel
-        // instance, no handle twice (its split-k words would be shared), and no output overlapping
-        // an input or output of another entry of the run, so that their order does not matter.
-        // Anything else goes through its own launch, in order.
-        lutgemm_kernels::MultiMatvecArgs multi{};
-        Range xr[lutgemm_kernels::kMaxFused], yr[lutgemm_kernels::kMaxFused];
-        const Shape *shapes[lutgemm_kernels::kMaxFused];
-        int rows_of[lutgemm_kernels::kMaxFused], slots[lutgemm_kernels::kMaxFused];
-        int j = i;
-        const lutgemm_weight *w0 = ws[i];
-        const int kind = w0 && xs[i] && ys[i] ? kind_of(w0, ms[i]) : 0;
-        for (; kind != 0 && j < count && j - i < lutgemm_kernels::kMaxFused; j++) {
-            const lutgemm_weight *w = ws[j];
-            if (!w || !xs[j] || !ys[j] || ((uintptr_t)xs[j] & 15u) != 0 || kind_of(w, ms[j]) != kind) break;
-            const Shape &s = w->shape;
-            if (s.q != w0->shape.q || s.has_offset != w0->shape.has_offset || s.gsub != w0->shape.gsub ||
-                w->device != w0->device)
-                break;
-            const int e = j - i;
-            xr[e] = Range{(uintptr_t)xs[j], (uintptr_t)xs[j] + (size_t)ms[j] * s.k * 2};
-            yr[e] = Range{(uintptr_t)ys[j], (uintptr_t)ys[j] + (size_t)ms[j] * s.n * 2};
-            bool independent = true;
-            for (int p = 0; p < e && independent; p++)
-                independent = ws[i + p] != w && !overlap(yr[e], yr[p]) && !overlap(yr[e], xr[p]) && !overlap(xr[e], yr[p]);
-            if (!independent) break;
-            shapes[e] = &s;
-            rows_of[e] = ms[j];
-            lutgemm_kernels::MatvecArgs &a = multi.entry[e];
-            a.signs = w->d_signs;
-            a.scales = w->d_scales;
-            a.k = s.k;
-            a.n = s.n;
-            a.ts = s.ts;
-            a.nb = s.nb;
-            a.x = xs[j];
-            a.y = ys[j];
-            a.y_stride = 1;
-            a.rows = ms[j];
-            a.x_row_stride = s.k;
-            a.y_row_stride = s.n;
-            a.accum_row_stride = (long long)s.nb * kBatch;
-        }
-        const int run = j - i;
-        if (run < 2) {
+        FusedRun run;
+        const int j = form_run(ws, xs, ys, ms, count, i, &run);
+        if (run.count < 2) {
             int st = run_matvec(ws[i], xs[i], ys[i], ms[i], stream, false, false);
             if (st != LUTGEMM_OK) return st;
             i++;
             continue;
         }
-        if (int st_dev = check_device(w0)) return st_dev;
-        const FusedPlan fp = kind == 2 ? choose_fused_batch_plan(shapes, rows_of, run, w0->compute_units)
-                                       : choose_fused_plan(shapes, run, w0->compute_units, kind == 1 ? 1 : 2);
-        int blocks = 0;
-        for (int e = 0; e < run; e++) {
-            lutgemm_kernels::MatvecArgs &a = multi.entry[e];
-            a.ntiles = div_up(a.nb, fp.waves);
-            a.blocks_per_split = fp.blocks_per_group < a.ts ? fp.blocks_per_group : a.ts;
-            a.k_splits = div_up(a.ts, a.blocks_per_split);
-            multi.first_block[e] = blocks;
-            blocks += a.ntiles * a.k_splits;
-            lutgemm_weight *we = const_cast<lutgemm_weight *>(ws[i + e]);
-            if (int st_ws = stream_set(we, stream, &slots[e])) return st_ws;
-            a.accum = we->set[slots[e]].accum;
-        }
-        multi.count = run;
-        hipError_t e = kind != 2 ? lutgemm_kernels::launch_matvec_multi(w0->shape.q, w0->shape.has_offset, w0->shape.gsub, multi,
-                                                                       blocks, fp.waves, static_cast<hipStream_t>(stream))
-                                 : lutgemm_kernels::launch_batch_multi(w0->shape.q, w0->shape.has_offset, w0->shape.gsub, multi,
-                                                                       blocks, fp.waves, static_cast<hipStream_t>(stream));
-        if (e != hipSuccess) return hip_fail(e, kind != 2 ? "launch lut_matvec_multi_kernel" : "launch lut_batch_multi_kernel");
-        for (int en = 0; en < run; en++) note_launch(const_cast<lutgemm_weight *>(ws[i + en]), slots[en], stream);
+        if (int st_dev = check_device(ws[i])) return st_dev;
+        FusedPlan fp;
+        if (!measured_fused_plan(run, &fp)) fp = model_fused_plan(run, nullptr);
+        if (int st = launch_run(run, fp, stream)) return st;
         i = j;
     }
+    return LUTGEMM_OK;
+}
+
+int lutgemm_matvec_many_autotune(const lutgemm_weight *const *ws, const void *const *xs, void *const *ys,
+                                 const int *ms, int count, void *stream)
+{
+    if (!ws || !xs || !ys || !ms) return fail(LUTGEMM_ERR_NULL_POINTER, "null argument to matvec_many_autotune");
+    if (count < 0) return fail(LUTGEMM_ERR_BAD_SHAPE, "count=%d is negative", count);
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    hipEvent_t e0 = nullptr, e1 = nullptr;
+    hipError_t he = hipEventCreate(&e0);
+    if (he == hipSuccess) he = hipEventCreate(&e1);
+    int status = he == hipSuccess ? LUTGEMM_OK : hip_fail(he, "hipEventCreate");
+    int i = 0;
+    while (status == LUTGEMM_OK && i < count) {
+        FusedRun run;
+        const int j = form_run(ws, xs, ys, ms, count, i, &run);
+        if (run.count < 2) {   // launched on its own: the handle's plan applies (lutgemm_weight_autotune)
+            status = run_matvec(ws[i], xs[i], ys[i], ms[i], stream, false, false);
+            i++;
+            continue;
+        }
+        status = check_device(ws[i]);
+        if (status != LUTGEMM_OK) break;
+        // the launch shapes the model ranks best, measured on the entries themselves
+        std::vector<FusedCandidate> cands;
+        const FusedPlan model = model_fused_plan(run, &cands);
+        std::sort(cands.begin(), cands.end(), [](const FusedCandidate &a, const FusedCandidate &b) { return a.cost < b.cost; });
+        // plans that differ only in k-blocks per workgroup beyond every entry's k-blocks are one launch shape
+        std::vector<FusedPlan> plans;
+        for (const FusedCandidate &c : cands) {
+            bool seen = false;
+            for (const FusedPlan &p : plans) seen = seen || same_launch(run, p, c.plan);
+            if (!seen) plans.push_back(c.plan);
+            if (plans.size() == kFusedCandidates) break;
+        }
+        auto time_plan = [&](const FusedPlan &p, int reps, float *us) -> int {
+            int stt = launch_run(run, p, stream);   // untimed: first touch of this shape
+            hipError_t e = hipEventRecord(e0, st);
+            for (int r = 0; r < reps && stt == LUTGEMM_OK; r++) stt = launch_run(run, p, stream);
+            if (stt != LUTGEMM_OK) return stt;
+            if (e == hipSuccess) e = hipEventRecord(e1, st);
+            if (e == hipSuccess) e = hipEventSynchronize(e1);
+            float ms_ = 0.f;
+            if (e == hipSuccess) e = hipEventElapsedTime(&ms_, e0, e1);
+            if (e != hipSuccess) return hip_fail(e, "fused autotune timing");
+            *us = ms_ * 1e3f / (float)reps;
+            return LUTGEMM_OK;
+        };
+        // clocks up first (the candidates measured first would look slow), then two sweeps, the
+        // minimum of which counts; the model's own choice is among the candidates (it ranks first)
+        {
+            const auto t0 = std::chrono::steady_clock::now();
+            float us = 0.f;
+            while (status == LUTGEMM_OK && std::chrono::duration<double>(std::chrono::steady_clock::now() - t0).count() < 0.03)
+                status = time_plan(model, 8, &us);
+        }
+        std::vector<float> best(plans.size(), 1e30f);
+        for (int sweep = 0; sweep < 3 && status == LUTGEMM_OK; sweep++)
+            for (size_t c = 0; c < plans.size() && status == LUTGEMM_OK; c++) {
+                float us = 0.f;
+                status = time_plan(plans[c], 6, &us);
+                if (status == LUTGEMM_OK && us < best[c]) best[c] = us;
+            }
+        if (status == LUTGEMM_OK) {
+            size_t pick = 0;
+            for (size_t c = 1; c < plans.size(); c++)
+                if (best[c] < best[pick]) pick = c;
+            remember_fused_plan(run, plans[pick]);
+        }
+        i = j;
+    }
+    if (e0) (void)hipEventDestroy(e0);
+    if (e1) (void)hipEventDestroy(e1);
+    return status;
+}
+
+int lutgemm_matvec_many_plan(const lutgemm_weight *const *ws, const void *const *xs, void *const *ys,
+                             const int *ms, int count, int *entries_in_first_launch, int *waves_per_group,
+                             int *k_blocks_per_group, int *measured)
+{
+    if (!ws || !xs || !ys || !ms) return fail(LUTGEMM_ERR_NULL_POINTER, "null argument to matvec_many_plan");
+    if (count < 1) return fail(LUTGEMM_ERR_BAD_SHAPE, "count=%d: no entry to plan", count);
+    FusedRun run;
+    form_run(ws, xs, ys, ms, count, 0, &run);
+    if (entries_in_first_launch) *entries_in_first_launch = run.count < 2 ? 1 : run.count;
+    FusedPlan fp{0, 0};
+    bool have = false;
+    if (run.count >= 2) {
+        have = measured_fused_plan(run, &fp);
+        if (!have) fp = model_fused_plan(run, nullptr);
+    }
+    if (waves_per_group) *waves_per_group = fp.waves;
+    if (k_blocks_per_group) *k_blocks_per_group = fp.blocks_per_group;
+    if (measured) *measured = have ? 1 : 0;
     return LUTGEMM_OK;
 }
 
@@ -1082,7 +1260,7 @@ int lutgemm_weight_plan_for(const lutgemm_weight *w, int m, int *workgroups, int
     if (m < 1 || m > LUTGEMM_MAX_BATCH)
         return fail(LUTGEMM_ERR_BAD_SHAPE, "m=%d outside 1..%d", m, LUTGEMM_MAX_BATCH);
     Plan p = m == 1 ? w->plan : w->plan2;
-    if (m >= 3 && batch_kernel_takes(w->shape)) {
+    if (m >= 3) {
         const int pass_rows = m < kRowsPerPass ? m : kRowsPerPass;
         p = w->batch_measured[pass_rows > 8] ? w->plan_batch[pass_rows > 8]
                                               : choose_batch_plan(w->shape, w->compute_units, pass_rows > 8 ? kRowsPerPass : 8);
@@ -1098,14 +1276,11 @@ int lutgemm_weight_set_batch_plan(lutgemm_weight *w, int waves_per_group, int k_
 {
     if (!w) return fail(LUTGEMM_ERR_NULL_POINTER, "null argument to weight_set_batch_plan");
     const Shape &s = w->shape;
-    if (!batch_kernel_takes(s))
-        return fail(LUTGEMM_ERR_UNSUPPORTED, "weights of more than %d planes do not go through the batch kernel",
-                    lutgemm_kernels::kBatchMaxPlanes);
     if (waves_per_group == 0 && k_splits == 0) {   // back to the model's choice
         w->batch_measured[0] = w->batch_measured[1] = false;
         return LUTGEMM_OK;
     }
-    const int wmax = lutgemm_kernels::batch_waves_max(s.gsub, s.qo);
+    const int wmax = lutgemm_kernels::batch_waves_max(s.gsub, s.q, s.qo);
     if (waves_per_group < lutgemm_kernels::kBatchWavesMin || waves_per_group > wmax)
         return fail(LUTGEMM_ERR_BAD_SHAPE, "waves_per_group=%d outside %d..%d", waves_per_group,
                     lutgemm_kernels::kBatchWavesMin, wmax);
@@ -1189,7 +1364,7 @@ int lutgemm_weight_autotune(lutgemm_weight *w, void *stream)
     void *x = nullptr, *y = nullptr;
     hipEvent_t e0 = nullptr, e1 = nullptr;
     int status = LUTGEMM_OK;
-    const size_t max_rows = batch_kernel_takes(s) ? (size_t)kRowsPerPass : (size_t)kTableRows;
+    const size_t max_rows = (size_t)kRowsPerPass;
     hipError_t e = hipMalloc(&x, max_rows * s.k * 2);
     if (e == hipSuccess) e = hipMalloc(&y, max_rows * s.n * 2);
     if (e == hipSuccess) e = hipMemsetAsync(x, 0, max_rows * s.k * 2, st);
@@ -1275,11 +1450,11 @@ int lutgemm_weight_autotune(lutgemm_weight *w, void *stream)
     // measured the same way.
     Plan chosen_batch[2] = {before_batch[0], before_batch[1]};
     bool have_batch[2] = {false, false};
-    for (int bi = 0; bi < 2 && batch_kernel_takes(s); bi++) {
+    for (int bi = 0; bi < 2; bi++) {
         const int rows = bi ? kRowsPerPass : 8;
         struct Timed { float ms; double cost; Plan p; };
         std::vector<Timed> timed;
-        for (int waves = lutgemm_kernels::kBatchWavesMin; waves <= lutgemm_kernels::batch_waves_max(s.gsub, s.qo); waves++)
+        for (int waves = lutgemm_kernels::kBatchWavesMin; waves <= lutgemm_kernels::batch_waves_max(s.gsub, s.q, s.qo); waves++)
             for (int ks = 1; ks <= s.ts && ks <= kMaxSplits; ks++) {
                 Plan p;
                 const double cost = batch_plan_cost(s, w->compute_units, waves, ks, rows, &p);

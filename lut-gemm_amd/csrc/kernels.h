@@ -56,9 +56,13 @@ hipError_t launch_matvec(int q, int has_offset, int gsub, const MatvecArgs &a, i
 hipError_t launch_matvec_multi(int q, int has_offset, int gsub, const MultiMatvecArgs &m, int workgroups, int waves,
                                hipStream_t stream);
 
-// 1..kBatchRows activation rows in one pass (matrix cores); up to kBatchMaxPlanes planes.  A workgroup has kBatchWavesMin .. kBatchWaves wavefronts:
-// wavefront w stages activation rows w and w + wavefronts, so eight cover the 16 rows of a pass.
-constexpr int kBatchMaxPlanes = 4;
+// 1..kBatchRows activation rows in one pass (matrix cores), any number of planes up to kBatchMaxPlanes.
+// A workgroup has kBatchWavesMin .. kBatchWaves wavefronts: wavefront w stages activation rows w and
+// w + wavefronts, so eight cover the 16 rows of a pass.  A tile of more than kBatchWidePlanes planes
+// needs more than 128 registers per lane, so such weights run with exactly kBatchWavesMin wavefronts
+// (which may then use 256 registers each).
+constexpr int kBatchMaxPlanes = 8;
+constexpr int kBatchWidePlanes = 4;
 constexpr int kBatchWaves = 16;
 constexpr int kBatchWavesMin = 8;
 // LDS of a workgroup of the batch kernel: two activation blocks of 17 rows of 2064 bytes (every
@@ -70,12 +74,13 @@ constexpr int batch_lds_bytes(int waves, int gsub, int qo)
 {
     return 2 * 17 * 2064 + waves * (1024 + batch_scale_area_bytes(gsub, qo));
 }
-constexpr int batch_waves_max(int gsub, int qo)
+constexpr int batch_waves_max(int gsub, int q, int qo)
 {
-    int w = kBatchWaves;
+    int w = q > kBatchWidePlanes ? kBatchWavesMin : kBatchWaves;
     while (w > kBatchWavesMin && batch_lds_bytes(w, gsub, qo) > 160 * 1024) w--;
     return w;
 }
+static_assert(batch_lds_bytes(kBatchWavesMin, 4, kBatchMaxPlanes + 1) <= 160 * 1024, "LDS of a compute unit");
 hipError_t launch_batch(int q, int has_offset, int gsub, const MatvecArgs &a, int workgroups, int waves, hipStream_t stream);
 // A work list of independent batches in one launch: entries sharing q, has_offset, gsub and the
 // wavefronts per workgroup, each with 1..kBatchRows rows and its own ntiles / k_splits / blocks_per_split;

@@ -32,6 +32,7 @@ EXPORTED = [
     "lutgemm_status_string", "lutgemm_version", "lutgemm_pack_file", "lutgemm_unpack_file", "lutgemm_weight_save",
     "lutgemm_weight_load", "lutgemm_weight_clone", "lutgemm_read_probe", "lutgemm_dense_gemv_f16",
     "lutgemm_weight_reset_workspace", "lutgemm_matvec_static", "lutgemm_matvec_each",
+    "lutgemm_matvec_many_autotune", "lutgemm_matvec_many_plan",
 ]
 
 
@@ -82,6 +83,8 @@ def load():
     L.lutgemm_matvec_static.argtypes = [vp, vp, vp, i, vp]
     L.lutgemm_matvec_many.argtypes = [vp, vp, vp, vp, i, vp]
     L.lutgemm_matvec_each.argtypes = [vp, vp, vp, vp, i, vp]
+    L.lutgemm_matvec_many_autotune.argtypes = [vp, vp, vp, vp, i, vp]
+    L.lutgemm_matvec_many_plan.argtypes = [vp, vp, vp, vp, i, pi, pi, pi, pi]
     L.lutgemm_dequantize.argtypes = [vp, vp, i, vp]
     L.lutgemm_weight_unpack.argtypes = [vp, vp, vp, vp]
     L.lutgemm_weight_plan.argtypes = [vp, pi, pi, pi, pi]
@@ -331,6 +334,17 @@ class MatvecSequence:
     def launch(self, stream=0, fused=True):
         fn = load().lutgemm_matvec_many if fused else load().lutgemm_matvec_each
         _check(fn(self._ws, self._xs, self._ys, self._ms, self.count, stream or None))
+
+    def autotune(self, stream=0):
+        """Measure the launch shapes of the fused launches of this list and remember the fastest for
+        every list of the same shapes (lutgemm_matvec_many_autotune)."""
+        _check(load().lutgemm_matvec_many_autotune(self._ws, self._xs, self._ys, self._ms, self.count, stream or None))
+
+    def fused_plan(self):
+        """Launch shape of the list's first launch: dict(entries, waves, k_blocks, measured)."""
+        v = [ctypes.c_int() for _ in range(4)]
+        _check(load().lutgemm_matvec_many_plan(self._ws, self._xs, self._ys, self._ms, self.count, *[ctypes.byref(x) for x in v]))
+        return dict(entries=v[0].value, waves=v[1].value, k_blocks=v[2].value, measured=bool(v[3].value))
 
 
 def read_probe(weights, stream=0):

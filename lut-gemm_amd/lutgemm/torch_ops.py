@@ -13,22 +13,26 @@ by all layers (one per device and stream), so a layer never holds more than its 
 `keep_dense=True` keeps a private dense copy instead (2 k n bytes) and skips the rebuild.  Up to
 the threshold the library streams the packed weight
 (one or two rows through the table-lookup kernels, more through the batch kernel, 16 rows per
-pass).  The default threshold depends on the weight (default_dense_threshold): it is where the
-two routes met when measured on MI355X.
+pass).  The default threshold depends on the weight and on keep_dense (default_dense_threshold):
+it is where the two routes met when measured on MI355X.
 """
 
 
-def default_dense_threshold(weight):
-    """Rows up to which the packed routes beat dequantised weight + library GEMM (measured on
-    MI355X at k = n = 12288 and k = 12288, n = 49152; LutLinear(dense_threshold=...) overrides).
+def default_dense_threshold(weight, keep_dense=False):
+    """Rows up to which the packed route beats dequantised weight + library GEMM (measured on MI355X
+    at k = n = 12288 and at k = 7168, n = 28672; LutLinear(dense_threshold=...) overrides).
 
-    Weights of up to four planes go through the batch kernel: one pass of 16 rows costs 21-49 us
-    (one to four planes, group sizes 128 down to 32) against 50 us for the GEMM, two passes 40-98 us
-    against 56 us: 32 rows for one or two planes, 16 for three or four.  More planes go through
-    two-row passes of the table-lookup kernel, which lose to the GEMM from three rows on."""
-    if weight.nb <= 4:
-        return 32 if weight.nb <= 2 else 16
-    return 2
+    A pass of the batch kernel over up to 16 rows costs 22 / 24 / 30 / 36 us for one to four planes
+    and 41 / 43 / 50 / 57 us for five to eight (k = n = 12288).  The dense route costs the
+    dequantisation (75 us up to four planes, 97-130 us for five to eight) plus the GEMM (50-56 us up
+    to 32 rows), so by default it only pays from the number of passes on that costs as much:
+    80 rows for one or two planes, 64 for three, 48 beyond.  A layer that keeps its dense copy
+    (keep_dense) pays the GEMM alone: 32 rows for one or two planes, 16 for three to seven, and
+    eight planes leave the packed route from three rows on (57 against 50 us)."""
+    q = weight.nb
+    if keep_dense:
+        return 32 if q <= 2 else 16 if q <= 7 else 2
+    return 80 if q <= 2 else 64 if q == 3 else 48
 
 
 import weakref
@@ -109,7 +113,7 @@ class LutLinear(torch.nn.Module):
             self.weight.autotune(torch.cuda.current_stream().cuda_stream)
         self.handle = register(self.weight)
         self.in_features, self.out_features = c["k"], c["n"]
-        self.dense_threshold = default_dense_threshold(self.weight) if dense_threshold is None else dense_threshold
+        self.dense_threshold = default_dense_threshold(self.weight, keep_dense) if dense_threshold is None else dense_threshold
         self._dense = None
         if bias is not None:
             self.register_buffer("bias", torch.as_tensor(bias).to(torch.float16).to(self.device))
@@ -128,7 +132,7 @@ class LutLinear(torch.nn.Module):
         self.handle = register(self.weight)
         self.in_features, self.out_features = self.weight.kSize, self.weight.mSize
         dt = kw.get("dense_threshold")
-        self.dense_threshold = default_dense_threshold(self.weight) if dt is None else dt
+        self.dense_threshold = default_dense_threshold(self.weight, self.keep_dense) if dt is None else dt
         self._dense = None
         if bias is not None:
             self.register_buffer("bias", torch.as_tensor(bias).to(torch.float16).to(self.device))

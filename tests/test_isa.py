@@ -11,20 +11,34 @@ import os
 import re
 import subprocess
 
+import pytest
+
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 CSRC = os.path.join(ROOT, "lut-gemm_amd", "csrc")
 
 
-import pytest
+SOURCES = [("batch.hip", "lut_batch_kernel", "10MatvecArgs"), ("batch_multi.hip", "lut_batch_multi_kernel", "15MultiMatvecArgs")]
 
 
-def kernels_of(tmp_path, source, kernel="lut_batch_kernel", args="10MatvecArgs"):
-    out = os.path.join(str(tmp_path), "out.s")
-    cmd = ["/opt/rocm/bin/hipcc", "-O3", "-std=c++17", "-fPIC", "--offload-arch=gfx950", "-Xclang", "-target-feature",
-           "-Xclang", "-packed-fp32-ops", "-Wno-unused-command-line-argument", "-I", CSRC, "-S", "--cuda-device-only",
-           "-o", out, os.path.join(CSRC, source)]
-    subprocess.run(cmd, check=True, stdout=subprocess.DEVNULL, stderr=subprocess.DEVNULL)
-    text = open(out).read()
+@pytest.fixture(scope="module")
+def assembly(tmp_path_factory):
+    """gfx950 assembly of the two translation units of the batch kernel, compiled side by side."""
+    out_dir = tmp_path_factory.mktemp("isa")
+    jobs = {}
+    for source, _, _ in SOURCES:
+        out = os.path.join(str(out_dir), source + ".s")
+        cmd = ["/opt/rocm/bin/hipcc", "-O3", "-std=c++17", "-fPIC", "--offload-arch=gfx950", "-Xclang", "-target-feature",
+               "-Xclang", "-packed-fp32-ops", "-Wno-unused-command-line-argument", "-I", CSRC, "-S", "--cuda-device-only",
+               "-o", out, os.path.join(CSRC, source)]
+        jobs[source] = (subprocess.Popen(cmd, stdout=subprocess.DEVNULL, stderr=subprocess.DEVNULL), out)
+    texts = {}
+    for source, (proc, out) in jobs.items():
+        assert proc.wait() == 0, source
+        texts[source] = open(out).read()
+    return texts
+
+
+def kernels_of(text, kernel, args):
     found = {}
     for m in re.finditer(r"^(_ZN\S*%s(\S*?)EEvNS_%sE):[^\n]*\n(.*?)s_endpgm" % (kernel, args), text, re.S | re.M):
         body = [ln.strip() for ln in m.group(3).splitlines() if ln.strip() and not ln.strip().startswith(";")]
@@ -101,19 +115,21 @@ def test_the_in_flight_check_sees_a_short_wait():
 MAX_SCRATCH_BYTES = 128
 
 
-@pytest.mark.parametrize("source,kernel,args", [("batch.hip", "lut_batch_kernel", "10MatvecArgs"),
-                                                ("batch_multi.hip", "lut_batch_multi_kernel", "15MultiMatvecArgs")])
-def test_batch_kernel_assembly(tmp_path, source, kernel, args):
-    kernels = kernels_of(tmp_path, source, kernel, args)
-    assert len(kernels) == 48, sorted(kernels)   # 4 plane counts x offset x 3 scale layouts x second staged row
+@pytest.mark.parametrize("source,kernel,args", SOURCES)
+def test_batch_kernel_assembly(assembly, source, kernel, args):
+    kernels = kernels_of(assembly[source], kernel, args)
+    # 4 plane counts x offset x 3 scale layouts x second staged row, and for 5 to 8 planes the one
+    # instantiation of eight wavefronts that stages two rows
+    assert len(kernels) == 48 + 24, sorted(kernels)
     for name, (body, meta) in sorted(kernels.items()):
         ops = [ln.split()[0] for ln in body]
-        q = int(re.match(r"ILi(\d)E", name).group(1))
+        q, offset, gsub, width, two = [int(v) for v in re.match(r"ILi(\d)ELb(\d)ELi(\d)ELi(\d+)ELb(\d)E", name).groups()]
         vgprs = int(re.search(r"\.amdhsa_next_free_vgpr (\d+)", meta).group(1))
-        assert vgprs <= 128, (name, vgprs)     # 16 wavefronts per workgroup fit a compute unit
+        # 16 wavefronts per workgroup fit a compute unit; more than four planes run with eight
+        assert vgprs <= (128 if q <= 4 else 256), (name, vgprs)
+        assert (width, two) == (8, 1) if q > 4 else width == 16, name
         assert ops.count("ds_read_b64_tr_b8") == 4 * q, name            # the transposition is the LDS's
-        offset = 1 if "ELb1ELi" in name[:12] else 0
-        groups_of_32 = "ELi4ELi16E" in name     # four scale groups per 128 k: the scales are the matrix operand, the offset term per output half
+        groups_of_32 = gsub == 4     # four scale groups per 128 k: the scales are the matrix operand, the offset term per output half
         assert ops.count("v_smfmac_f32_16x16x64_f16") == 32 * q + (32 if groups_of_32 else 16) * offset, name
         assert ops.count("v_and_or_b32") >= 16 * q, name                  # the index of a step: one instruction per sign word and parity
         assert "v_cvt_f32_f16_e32" not in ops, name                       # scales applied without conversions

@@ -112,14 +112,18 @@ def test_operator_argument_checks(lutgemm, device):
 
 
 def test_default_dense_threshold_follows_the_weight(lutgemm, device):
-    """Weights the batch kernel takes (up to four planes) keep the packed route for one or two
-    passes of 16 rows, the others leave it from three rows on."""
+    """The packed route is kept for as many passes of 16 rows as cost less than the dense route:
+    more of them when the dense weight has to be rebuilt per call than when the layer keeps it."""
     from lutgemm import quantize, torch_ops
     print("case default dense threshold", flush=True)
     lin, _ = _layer(5, out_f=64, in_f=512, bias=False)
-    for qbits, g, want in ((2, 128, 32), (4, 128, 16), (3, 64, 16), (1, 32, 32), (5, 128, 2)):
+    for qbits, g, want, want_kept in ((2, 128, 80, 32), (4, 128, 48, 16), (3, 64, 64, 16), (1, 32, 80, 32), (5, 128, 48, 16),
+                                      (8, 128, 48, 2)):
         c, _ = quantize.quantize_linear(lin.weight.detach(), qbits, g, "rtn", rounds=0)
         layer = torch_ops.LutLinear(c)
         assert layer.dense_threshold == want, (qbits, g, layer.dense_threshold)
+        kept = torch_ops.LutLinear(c, keep_dense=True)
+        assert kept.dense_threshold == want_kept, (qbits, g, kept.dense_threshold)
+        kept.weight.close()
         assert torch_ops.LutLinear(c, dense_threshold=7).dense_threshold == 7
         layer.weight.close()
