@@ -389,7 +389,10 @@ def run_cfg3(args, lutgemm, synth, torch, dev, stream):
     points = []
     tot_bytes = tot_us = tot_fused = 0.0
     worst = 0.0
-    for c in synth.CFG3_POINTS:
+    todo = [c for c in synth.CFG3_POINTS if args.point is None or (c["q"], c["g"]) == args.point]
+    if not todo:
+        sys.exit("bench.py: --point %s is not one of the cfg3 points" % (args.point,))
+    for c in todo:
         pt = Point(lutgemm, synth, torch, dev, c["k"], c["n"], c["q"], c["g"], False, 1, c["q"] * 10000 + c["g"],
                    stream.cuda_stream)
         us, us_hot = time_point(lutgemm, torch, stream, pt, args.steps, args.warmup)
@@ -404,7 +407,7 @@ def run_cfg3(args, lutgemm, synth, torch, dev, stream):
     value = tot_bytes / tot_us / 1e3
     fused = tot_bytes / tot_fused / 1e3
     line = base_line(args, "weight-GB/s over the k=n=7168 sweep (q 1..4 x g 32,64,128,k), m=1 fp16", value,
-                     tot_us / len(points), "cfg3: 16 BCQ matvecs k=n=7168, q in 1..4, g in {32,64,128,7168}",
+                     tot_us / len(points), "cfg3: %d BCQ matvecs k=n=7168, q in 1..4, g in {32,64,128,7168}" % len(points),
                      {"points": len(points),
                       "launch": "per point, bursts with one kernel launch per matvec (one weight copy each), back to back"})
     line["ms_per_step"] = tot_us / 1e3
@@ -416,7 +419,7 @@ def run_cfg3(args, lutgemm, synth, torch, dev, stream):
                         "frac": value / HBM_PEAK_GBS, "traffic": None, "kernel": "lut_matvec_kernel<q,false,gsub>",
                         "value_is": "back_to_back", "frac_back_to_back": value / HBM_PEAK_GBS,
                         "frac_fused_independent": fused / HBM_PEAK_GBS,
-                        "note": "aggregate packed-weight bytes / summed time over the 16 points"}
+                        "note": "aggregate packed-weight bytes / summed time over the %d points" % len(points)}
     line["cpu_baseline"] = None
     return line
 
@@ -573,6 +576,7 @@ def main():
     ap.add_argument("--copies", type=int, default=33, help="cfg1: distinct weight copies rotated through")
     ap.add_argument("--plan", default=None,
                     help="cfg0/1/2: WAVES,KSPLITS launch plan instead of the measured choice (profiling runs)")
+    ap.add_argument("--point", default=None, help="cfg3: only the point Q,G of the sweep (profiling runs)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-dense", action="store_true", help="skip the dense fp16 GEMV comparator")
     ap.add_argument("--copy-calibration", action="store_true",
@@ -580,6 +584,8 @@ def main():
     args = ap.parse_args()
     if args.plan:
         args.plan = tuple(int(v) for v in args.plan.split(","))
+    if args.point:
+        args.point = tuple(int(v) for v in args.point.split(","))
     if args.gpus != 1:
         sys.exit("bench.py: this build measures one GPU only (got --gpus %d); a matvec shards by output "
                  "columns, no multi-GPU path is built" % args.gpus)
