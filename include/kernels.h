@@ -1,6 +1,7 @@
 // kernels.h -- the matmul entry points of the reference's C++ API (lutGEMM/include/kernels.h:26-33),
-// header only, on top of the C ABI of this library.  Every batch size stays on the table-lookup
-// kernel (the reference dequantises and calls a dense GEMM for m > 1, lutGEMM/src/kernels.cu:73-79),
+// header only, on top of the C ABI of this library.  Every batch size streams the packed weight (one
+// and two rows through the table-lookup kernels, three and more through the batch kernel, 16 rows per
+// pass; the reference dequantises and calls a dense GEMM for m > 1, lutGEMM/src/kernels.cu:73-79),
 // the offset is applied for every m, no memset of the output is needed, and `algo` is accepted
 // and ignored exactly as in the reference (mv_fp16.hpp:121).  Work is issued on the default stream
 // and is asynchronous, as in the reference; failures throw std::runtime_error.

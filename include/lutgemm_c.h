@@ -157,7 +157,8 @@ int lutgemm_matvec_many(const lutgemm_weight *const *ws, const void *const *xs, 
  * launch shapes (wavefronts per workgroup, k-blocks per workgroup) the cost model ranks best, the
  * model's own choice among them, with the entries themselves on `stream` (a few launches each; ys
  * receive valid results; the device is kept busy for 30 ms first so that the clocks are up) and
- * remembers the fastest, process-wide, under the shapes of the run: kernel instance, compute units,
+ * remembers the fastest (the model's choice unless another shape measured at least 2 % faster),
+ * process-wide, under the shapes of the run: kernel instance, compute units,
  * and (k, n, rows) of its entries in order.  From then on every lutgemm_matvec_many run of those
  * shapes, whatever its handles and buffers, is launched that way.  The constants of the cost model
  * were fitted on one MI355X; this call is how a caller checks them on the box it runs on.
