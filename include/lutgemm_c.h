@@ -97,9 +97,11 @@ int lutgemm_weight_info(const lutgemm_weight *w, lutgemm_weight_info_t *info);
  * the same tolerance, but a row may differ in the last bit from its own one-row call (another order
  * of the fp32 additions).
  * Launches on one stream run one after the other and share one set of split-k accumulators of the
- * handle; every further stream that launches on the handle gets a set of its own (allocated at that
- * stream's first launch, so not under graph capture), so launches on different streams may overlap
- * in time.  A handle keeps four sets.  A fifth stream takes over the set of the stream that used
+ * handle; every further stream that launches on the handle gets a set of its own, allocated at that
+ * stream's first launch, so launches on different streams may overlap in time.  A first launch
+ * under graph capture is refused with LUTGEMM_ERR_UNSUPPORTED before anything is allocated (launch
+ * once on the stream before capturing), as are the calls that synchronise: the two autotune calls
+ * and lutgemm_weight_reset_workspace.  A handle keeps four sets.  A fifth stream takes over the set of the stream that used
  * the handle least recently: at once if that stream's launches on the handle have completed,
  * otherwise the new stream is made to wait for them (hipStreamWaitEvent) first; to know, every
  * launch records an event once a handle serves more than one stream.  Launches issued under graph

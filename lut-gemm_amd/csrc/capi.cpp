@@ -303,6 +303,23 @@ int check_device(const lutgemm_weight *w)
 
 size_t set_words(const lutgemm_weight *w) { return (size_t)kRowsPerPass * w->shape.nb * kBatch; }
 
+// Work of `stream` is being recorded into a graph: nothing may allocate, synchronise or time there.
+bool stream_capturing(void *stream)
+{
+    hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(static_cast<hipStream_t>(stream), &capturing) != hipSuccess) {
+        (void)hipGetLastError();
+        return false;
+    }
+    return capturing != hipStreamCaptureStatusNone;
+}
+
+int refuse_capture(void *stream, const char *what)
+{
+    if (!stream_capturing(stream)) return LUTGEMM_OK;
+    return fail(LUTGEMM_ERR_UNSUPPORTED, "%s synchronises with the device and cannot run on a stream under graph capture", what);
+}
+
 // Device memory of set i (idempotent).  Allocates: not for a stream that is being captured.
 int alloc_set(lutgemm_weight *w, int i)
 {
@@ -350,6 +367,11 @@ int stream_set(lutgemm_weight *w, void *stream, int *slot)
     int take = -1;
     if (w->slots_used < kStreamSlots) {
         take = w->slots_used;
+        if ((!w->set[take].accum || !w->set[take].xrows) && stream_capturing(stream))
+            return fail(LUTGEMM_ERR_UNSUPPORTED,
+                        "the first launch of a stream on this handle allocates the stream's split-k words, which "
+                        "graph capture forbids: launch once on the stream before capturing, or capture "
+                        "lutgemm_matvec_static");
         if (int st = alloc_set(w, take)) return st;
         if (!w->set[take].done) {
             hipError_t e = hipEventCreateWithFlags(&w->set[take].done, hipEventDisableTiming);
@@ -628,6 +650,10 @@ int run_matvec(const lutgemm_weight *w, const void *x, void *y, int m, void *str
         // staging rows belong to the stream's set, or, for the allocation-free entry point, to set 0
         StreamSet &t = mw->set[slot];
         if (m > t.xrows_cols) {
+            if (stream_capturing(stream))
+                return fail(LUTGEMM_ERR_UNSUPPORTED,
+                            "m=%d columns need larger staging rows than the stream's set holds (%d), and graph capture "
+                            "forbids the allocation: call once with this m before capturing", m, t.xrows_cols);
             // earlier launches of this stream may still read the old buffer
             hipError_t e = hipStreamSynchronize(st);
             if (e != hipSuccess) return hip_fail(e, "hipStreamSynchronize");
@@ -1005,6 +1031,7 @@ int lutgemm_weight_reset_workspace(lutgemm_weight *w, void *stream)
 {
     if (!w) return fail(LUTGEMM_ERR_NULL_POINTER, "null argument to weight_reset_workspace");
     if (int st_dev = check_device(w)) return st_dev;
+    if (int st_cap = refuse_capture(stream, "lutgemm_weight_reset_workspace")) return st_cap;
     std::lock_guard<std::mutex> lock(w->slot_mutex);
     hipError_t e = hipDeviceSynchronize();  // no launch may still be using the words
     if (e != hipSuccess) return hip_fail(e, "hipDeviceSynchronize");
@@ -1067,6 +1094,7 @@ int lutgemm_matvec_many_autotune(const lutgemm_weight *const *ws, const void *co
 {
     if (!ws || !xs || !ys || !ms) return fail(LUTGEMM_ERR_NULL_POINTER, "null argument to matvec_many_autotune");
     if (count < 0) return fail(LUTGEMM_ERR_BAD_SHAPE, "count=%d is negative", count);
+    if (int st_cap = refuse_capture(stream, "lutgemm_matvec_many_autotune")) return st_cap;
     hipStream_t st = static_cast<hipStream_t>(stream);
     hipEvent_t e0 = nullptr, e1 = nullptr;
     hipError_t he = hipEventCreate(&e0);
@@ -1324,6 +1352,7 @@ int lutgemm_weight_autotune(lutgemm_weight *w, void *stream)
 {
     if (!w) return fail(LUTGEMM_ERR_NULL_POINTER, "null argument to weight_autotune");
     if (int st_dev = check_device(w)) return st_dev;
+    if (int st_cap = refuse_capture(stream, "lutgemm_weight_autotune")) return st_cap;
     const Shape &s = w->shape;
     hipStream_t st = static_cast<hipStream_t>(stream);
     // candidates: the best plans of the model, measured on the device

@@ -807,6 +807,65 @@ def test_one_handle_on_many_streams(lutgemm, oracle, device):
     W.close()
 
 
+def test_graph_capture_refuses_what_allocates_or_synchronises(lutgemm, oracle, device):
+    """Under graph capture a stream's first launch on a handle (it would allocate the stream's set),
+    the autotune calls and the workspace reset return LUTGEMM_ERR_UNSUPPORTED before any HIP call
+    that would invalidate the capture; the capture itself stays usable, and after one launch outside
+    capture the same stream captures and replays the matvec bit for bit."""
+    import torch
+    from lutgemm import synth
+    k, n, q, g = 2048, 1024, 3, 128
+    w, W = make(lutgemm, synth, k, n, q, g, seed=19)
+    _, W2 = make(lutgemm, synth, k, n, q, g, seed=20)
+    x = torch.from_numpy(synth.make_x(1, k, seed=19)).to(device)
+    want = torch.zeros((1, n), dtype=torch.float16, device=device)
+    W.matvec(x.data_ptr(), want.data_ptr(), 1, torch.cuda.current_stream().cuda_stream)   # set 0 serves this stream
+    torch.cuda.synchronize()
+    assert_within_tolerance(want.cpu().numpy(), truth_of(oracle, w, x.cpu().numpy()), "eager")
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    out = torch.zeros_like(want)
+    out2 = torch.zeros_like(want)
+    seq = lutgemm.MatvecSequence([(W, x.data_ptr(), out.data_ptr(), 1), (W2, x.data_ptr(), out2.data_ptr(), 1)])
+    refused = []
+    graph = torch.cuda.CUDAGraph()
+    say("case capture: refused calls")
+    with torch.cuda.stream(side):
+        sh = side.cuda_stream
+        with torch.cuda.graph(graph, stream=side):
+            out2.mul_(1.0)   # the graph holds one ordinary kernel
+            for call in (lambda: W.matvec(x.data_ptr(), out.data_ptr(), 1, sh), lambda: W.autotune(sh),
+                         lambda: W.reset_workspace(sh), lambda: seq.autotune(sh)):
+                try:
+                    call()
+                    refused.append(0)
+                except lutgemm.LutGemmError as e:
+                    refused.append(e.status)
+    torch.cuda.synchronize()
+    assert refused == [lutgemm.ERR_UNSUPPORTED] * 4, refused
+    graph.replay()
+    torch.cuda.synchronize()
+    say("case capture: after a launch outside capture")
+    with torch.cuda.stream(side):
+        W.matvec(x.data_ptr(), out.data_ptr(), 1, side.cuda_stream)
+        side.synchronize()
+        assert torch.equal(out, want)
+        out.zero_()
+        side.synchronize()
+        graph2 = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph2, stream=side):
+            W.matvec(x.data_ptr(), out.data_ptr(), 1, side.cuda_stream)
+    torch.cuda.synchronize()
+    for rep in range(3):
+        out.zero_()
+        torch.cuda.synchronize()
+        graph2.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out, want), "replay %d" % rep
+    W.close()
+    W2.close()
+
+
 def test_dense_gemv_comparator(lutgemm, device):
     """The plain streaming fp16 GEMV that the benchmark times next to the LUT kernel: fp32
     accumulation over fp16 inputs, rows whose length is not a multiple of the unrolled step, more
