@@ -1,6 +1,7 @@
 """GPU parity at the benchmark's real shapes: cfg2 (k=12288, n=49152, q=4, offset), the sixteen
 cfg3 points (k=n=7168) and the four cfg4 decoder-layer shapes with m in {1, 2, 4, 8} (FC2 has
-k=49152 = 96 k-blocks, also run with 96 k-splits).
+k=49152 = 96 k-blocks, also run with 96 k-splits), and shapes at the ends of the range: one k-block
+against 300,001 outputs, 256 k-blocks against 96 outputs or a single one.
 
 The HIP path computes the whole problem.  Output columns are independent, so the oracle
 (double accumulation over the fp16-rounded inputs) is evaluated on a strided subset of columns
@@ -130,4 +131,27 @@ def test_cfg4_full_size_all_batches(lutgemm, oracle, device, layer):
                 rows_m1 = y
         assert rows_m1 is not None
     check_unit_rows(lutgemm, oracle, device, w, W, [k - 1], cols, "cfg4 %s" % layer)
+    W.close()
+
+
+@pytest.mark.parametrize("k,n,q,g,offset", [
+    (32, 300001, 3, 32, True),        # a single ragged k-block, 9,376 output batches
+    (131072, 96, 8, 128, False),      # 256 k-blocks, three output batches, eight planes
+    (98304, 1, 2, 64, True),          # a single output
+    (64, 70000, 8, 64, True),
+])
+def test_extreme_aspect_ratios(lutgemm, oracle, device, k, n, q, g, offset):
+    """Very wide and very deep weights, every kernel family (one row, two rows, the batch kernel in
+    one and in two passes), rows and columns entry; the whole output is compared with the oracle."""
+    from lutgemm import synth
+    w = synth.make_weight(k, n, q, g, offset=offset, seed=k % 1000 + n % 1000)
+    W = lutgemm.BCQWeight(w["bW"], w["alpha"], k, n, q, k // g, w["q_bias"])
+    cols = np.arange(n)
+    for m in (1, 2, 5, 19):
+        say("case extreme", k, n, q, g, offset, "m", m, W.plan(m))
+        x = synth.make_x(m, k, seed=m)
+        truth = truth_on(oracle, w, x, cols)
+        for by_cols in (False, True):
+            y = run_matvec(lutgemm, W, x, device, cols=by_cols)
+            assert_within_tolerance(y, truth, "k=%d n=%d q=%d m=%d cols=%s" % (k, n, q, m, by_cols))
     W.close()
