@@ -550,6 +550,8 @@ def run_dequant(args, lutgemm, synth, torch, dev, stream):
         shapes.append(rec)
         W.close()
         del outs
+    if args.copy_calibration:
+        copy_calibration(torch, dev)
     head = shapes[0]["W[n][k]"]
     line = base_line(args, "GB/s of dequantisation to dense fp16 (packed tiles read + 2kn written), cfg1 weight, W[n][k]",
                      head["GBps"], head["us"], "dequantize: cfg1 weight k=n=12288 q=3 g=128 to fp16 W[n][k]", {})

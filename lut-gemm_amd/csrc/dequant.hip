@@ -171,18 +171,21 @@ __global__ __launch_bounds__(512) void dequantize_rows_kernel(DequantArgs a)
         const unsigned char *sp =
             a.signs + (tile * (size_t)(2 * Q) + h) * kUnitBytes + lane * 16 + (st & 1) * 8;
         const uint32_t *cp = reinterpret_cast<const uint32_t *>(a.scales) + (tile * kLanes + lane) * (size_t)(GSUB * QO);
+        // Ordinary loads, not streaming ones: the two wavefronts of a half read the two 8-byte halves of the
+        // same lines, and the four wavefronts of a batch the same scale words; the later ones should find
+        // them in the cache.
         // the 8 sign bytes of this quarter sit in .x/.y (first 8 outputs of the half) or .z/.w
         u32x4 sgh[Q];
 #pragma unroll
         for (int b = 0; b < Q; b++) {
-            const uint64_t v = __builtin_nontemporal_load(reinterpret_cast<const uint64_t *>(sp + (size_t)(2 * b) * kUnitBytes));
+            const uint64_t v = *reinterpret_cast<const uint64_t *>(sp + (size_t)(2 * b) * kUnitBytes);
             sgh[b].x = sgh[b].z = (uint32_t)v;
             sgh[b].y = sgh[b].w = (uint32_t)(v >> 32);
         }
         float sc[2 * GSUB * QO];  // [slot][plane or offset]
 #pragma unroll
         for (int d = 0; d < GSUB * QO; d++) {
-            const uint32_t rec = __builtin_nontemporal_load(cp + d);
+            const uint32_t rec = cp[d];
             const __half2 h2 = *reinterpret_cast<const __half2 *>(&rec);
             sc[2 * d] = __low2float(h2);
             sc[2 * d + 1] = __high2float(h2);
