@@ -107,8 +107,10 @@ int lutgemm_weight_info(const lutgemm_weight *w, lutgemm_weight_info_t *info);
  * launch records an event once a handle serves more than one stream.  Launches issued under graph
  * capture are not tracked, and a set last used that way is never handed on
  * (LUTGEMM_ERR_UNSUPPORTED if no set can be taken over; lutgemm_weight_clone gives further streams
- * handles of their own).  Launches from different host threads on the SAME stream must be serialised
- * by the caller, as for any stream.
+ * handles of their own).  Host threads may call on one handle at the same time as long as each uses a
+ * stream of its own (a set that a call has claimed is not handed to another stream before the call has
+ * issued its launches); launches from different host threads on the SAME stream must be serialised by
+ * the caller, as for any stream.
  * Non-finite values follow IEEE arithmetic whatever the launch plan: a NaN activation gives NaN
  * outputs, infinite partial sums give an infinity of their sign, or NaN if both signs occur.  With
  * more than one k-split the partial sums are added as fixed-point integers (2^-24 resolution);

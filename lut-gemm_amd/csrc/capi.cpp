@@ -15,6 +15,7 @@
 #include <map>
 #include <mutex>
 #include <new>
+#include <thread>
 #include <vector>
 
 #include "kernels.h"
@@ -74,6 +75,7 @@ struct StreamSet {
     hipEvent_t done;             // recorded behind the set's latest launch (only while done_valid)
     bool done_valid;
     unsigned long long last_use;
+    int leases;                  // calls that have claimed the set and not yet issued all their launches
 };
 
 struct lutgemm_weight {
@@ -354,13 +356,17 @@ size_t workspace_bytes(const lutgemm_weight *w)
     return bytes;
 }
 
-// The set launches on `stream` use.  The first launch of a stream on this handle claims one.
-int stream_set(lutgemm_weight *w, void *stream, int *slot)
+// The set launches on `stream` use.  The first launch of a stream on this handle claims one.  The
+// caller holds the set (a lease) until release_set: launches are issued outside the lock, and a set
+// that another host thread is about to launch on must not be handed to a further stream meanwhile.
+int stream_set_once(lutgemm_weight *w, void *stream, int *slot, bool *leased_elsewhere)
 {
+    *leased_elsewhere = false;
     std::lock_guard<std::mutex> lock(w->slot_mutex);
     for (int i = 0; i < w->slots_used; i++)
         if (w->set[i].stream == stream) {
             w->set[i].last_use = ++w->use_clock;
+            w->set[i].leases++;
             *slot = i;
             return LUTGEMM_OK;
         }
@@ -381,11 +387,12 @@ int stream_set(lutgemm_weight *w, void *stream, int *slot)
     } else {
         // all sets serve a stream: take over the least recently used one whose latest launch is known to
         // have completed; failing that, the least recently used one with a recorded event, after making
-        // `stream` wait for it
+        // `stream` wait for it.  A set under lease is not a candidate.
         int idle = -1, busy = -1;
         for (int i = 0; i < kStreamSlots; i++) {
             const StreamSet &t = w->set[i];
-            if (!t.done_valid) continue;
+            if (t.leases > 0) *leased_elsewhere = true;
+            if (!t.done_valid || t.leases > 0) continue;
             if (hipEventQuery(t.done) == hipSuccess) {
                 if (idle < 0 || t.last_use < w->set[idle].last_use) idle = i;
             } else if (busy < 0 || t.last_use < w->set[busy].last_use) {
@@ -407,18 +414,33 @@ int stream_set(lutgemm_weight *w, void *stream, int *slot)
     w->set[take].stream = stream;
     w->set[take].done_valid = false;
     w->set[take].last_use = ++w->use_clock;
+    w->set[take].leases = 1;
     *slot = take;
     return LUTGEMM_OK;
 }
 
-// Behind a launch on set `slot`: once the handle serves more than one stream, remember where the
-// stream stands, so that the set can be handed to another stream later.  A stream under capture
-// records nothing (the event would belong to the graph); its set is then not handed on.
-void note_launch(lutgemm_weight *w, int slot, void *stream)
+int stream_set(lutgemm_weight *w, void *stream, int *slot)
+{
+    // A lease lasts as long as another host thread needs to issue its launches: when that is all that
+    // stands in the way of a take-over, try again shortly instead of failing.
+    for (int attempt = 0;; attempt++) {
+        bool leased_elsewhere = false;
+        const int st = stream_set_once(w, stream, slot, &leased_elsewhere);
+        if (st != LUTGEMM_ERR_UNSUPPORTED || !leased_elsewhere || attempt >= 200000) return st;
+        std::this_thread::yield();
+    }
+}
+
+// End of a lease.  `launched`: the call has issued work on the set.  Once the handle serves more than
+// one stream, remember where the stream stands, so that the set can be handed to another stream later.
+// A stream under capture records nothing (the event would belong to the graph); its set is then not
+// handed on.
+void release_set(lutgemm_weight *w, int slot, void *stream, bool launched)
 {
     std::lock_guard<std::mutex> lock(w->slot_mutex);
-    if (w->slots_used < 2) return;
     StreamSet &t = w->set[slot];
+    if (t.leases > 0) t.leases--;
+    if (!launched || w->slots_used < 2) return;
     hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
     if (hipStreamIsCapturing(static_cast<hipStream_t>(stream), &capturing) != hipSuccess ||
         capturing != hipStreamCaptureStatusNone) {
@@ -428,6 +450,20 @@ void note_launch(lutgemm_weight *w, int slot, void *stream)
     }
     t.done_valid = hipEventRecord(t.done, static_cast<hipStream_t>(stream)) == hipSuccess;
 }
+
+struct SetLease {
+    lutgemm_weight *w = nullptr;
+    int slot = 0;
+    void *stream = nullptr;
+    bool launched = false;
+    SetLease() = default;
+    SetLease(const SetLease &) = delete;
+    SetLease &operator=(const SetLease &) = delete;
+    ~SetLease()
+    {
+        if (w) release_set(w, slot, stream, launched);
+    }
+};
 
 // The allocation-free entry point marks a device whose static split-k words a failed call may
 // have left non-zero; the next call on that device clears them first.
@@ -626,6 +662,7 @@ int run_matvec(const lutgemm_weight *w, const void *x, void *y, int m, void *str
         return fail(LUTGEMM_ERR_BAD_SHAPE, "x must be 16-byte aligned");
     hipStream_t st = static_cast<hipStream_t>(stream);
     int slot = 0;
+    SetLease lease;   // ends when this call returns
     if (static_ws) {
         const size_t words = lutgemm_kernels::kStaticSplitKWords;
         if ((size_t)kRowsPerPass * s.nb * kBatch > words)
@@ -643,6 +680,9 @@ int run_matvec(const lutgemm_weight *w, const void *x, void *y, int m, void *str
         }
     } else {
         if (int st_ws = stream_set(mw, stream, &slot)) return st_ws;
+        lease.w = mw;
+        lease.slot = slot;
+        lease.stream = stream;
         a.accum = mw->set[slot].accum;
     }
     if (cols && m > 1) {
@@ -668,6 +708,7 @@ int run_matvec(const lutgemm_weight *w, const void *x, void *y, int m, void *str
         uint16_t *rows = static_cast<uint16_t *>(t.xrows);
         hipError_t e = lutgemm_kernels::launch_gather_columns(x, rows, s.k, m, st);
         if (e != hipSuccess) return hip_fail(e, "launch gather_columns_kernel");
+        lease.launched = true;
         xh = rows;
     }
     a.x_row_stride = s.k;
@@ -697,8 +738,8 @@ int run_matvec(const lutgemm_weight *w, const void *x, void *y, int m, void *str
                 if (static_ws && r > 0) g_static_dirty[w->device] = true;
                 return hip_fail(e, "launch lut_batch_kernel");
             }
+            lease.launched = true;
         }
-        if (!static_ws) note_launch(mw, slot, stream);
         return LUTGEMM_OK;
     }
     // two activation rows per pass over the weight, a last single row if m is odd
@@ -724,8 +765,8 @@ int run_matvec(const lutgemm_weight *w, const void *x, void *y, int m, void *str
             if (static_ws && r > 0) g_static_dirty[w->device] = true;
             return hip_fail(e, "launch lut_matvec_kernel");
         }
+        lease.launched = true;
     }
-    if (!static_ws) note_launch(mw, slot, stream);
     return LUTGEMM_OK;
 }
 
@@ -857,6 +898,7 @@ int launch_run(FusedRun &run, const FusedPlan &fp, void *stream)
 {
     const Shape &s0 = *run.shape[0];
     int slots[lutgemm_kernels::kMaxFused];
+    SetLease leases[lutgemm_kernels::kMaxFused];   // end when this call returns
     int blocks = 0;
     for (int e = 0; e < run.count; e++) {
         lutgemm_kernels::MatvecArgs &a = run.multi.entry[e];
@@ -867,6 +909,9 @@ int launch_run(FusedRun &run, const FusedPlan &fp, void *stream)
         blocks += a.ntiles * a.k_splits;
         lutgemm_weight *we = const_cast<lutgemm_weight *>(run.handle[e]);
         if (int st_ws = stream_set(we, stream, &slots[e])) return st_ws;
+        leases[e].w = we;
+        leases[e].slot = slots[e];
+        leases[e].stream = stream;
         a.accum = we->set[slots[e]].accum;
     }
     run.multi.count = run.count;
@@ -875,7 +920,7 @@ int launch_run(FusedRun &run, const FusedPlan &fp, void *stream)
                                  : lutgemm_kernels::launch_batch_multi(s0.q, s0.has_offset, s0.gsub, run.multi, blocks, fp.waves,
                                                                        static_cast<hipStream_t>(stream));
     if (e != hipSuccess) return hip_fail(e, run.kind != 2 ? "launch lut_matvec_multi_kernel" : "launch lut_batch_multi_kernel");
-    for (int en = 0; en < run.count; en++) note_launch(const_cast<lutgemm_weight *>(run.handle[en]), slots[en], stream);
+    for (int en = 0; en < run.count; en++) leases[en].launched = true;
     return LUTGEMM_OK;
 }
 

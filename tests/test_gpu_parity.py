@@ -811,6 +811,56 @@ def test_one_handle_on_many_streams(lutgemm, oracle, device):
     W.close()
 
 
+def test_one_handle_from_many_host_threads(lutgemm, oracle, device):
+    """Eight host threads, each with a stream of its own, launch on one handle at the same time (the
+    binding releases the interpreter lock during a call): a set that one thread has claimed and is
+    launching on is not handed to another thread's stream in between, so every result equals the
+    same launch issued alone, whatever the row count (table-lookup, two-row and batch kernels)."""
+    import threading
+    import torch
+    from lutgemm import synth
+    k, n, q, g = 4096, 2048, 3, 128
+    w, W = make(lutgemm, synth, k, n, q, g, seed=21)
+    xs = synth.make_x(5, k, seed=21)
+    xd = torch.from_numpy(xs).to(device)
+    st = torch.cuda.current_stream().cuda_stream
+    want = {}
+    for m in (1, 2, 5):
+        y = torch.zeros((m, n), dtype=torch.float16, device=device)
+        W.matvec(xd.data_ptr(), y.data_ptr(), m, st)
+        torch.cuda.synchronize()
+        want[m] = y
+    assert_within_tolerance(want[5].cpu().numpy(), truth_of(oracle, w, xs), "serial")
+    threads, per_thread = 8, 120
+    streams = [torch.cuda.Stream() for _ in range(threads)]
+    rows = [[(1, 2, 5)[(t + i) % 3] for i in range(per_thread)] for t in range(threads)]
+    outs = [[torch.zeros((m, n), dtype=torch.float16, device=device) for m in rows[t]] for t in range(threads)]
+    torch.cuda.synchronize()
+    errors = []
+    go = threading.Barrier(threads)
+
+    def work(t):
+        try:
+            go.wait()
+            for m, y in zip(rows[t], outs[t]):
+                W.matvec(xd.data_ptr(), y.data_ptr(), m, streams[t].cuda_stream)
+        except Exception as e:   # reported by the main thread
+            errors.append((t, repr(e)))
+
+    say("case eight host threads on one handle")
+    pool = [threading.Thread(target=work, args=(t,)) for t in range(threads)]
+    for th in pool:
+        th.start()
+    for th in pool:
+        th.join()
+    torch.cuda.synchronize()
+    assert not errors, errors
+    for t in range(threads):
+        for i, (m, y) in enumerate(zip(rows[t], outs[t])):
+            assert torch.equal(y, want[m]), "thread %d launch %d (%d rows) differs" % (t, i, m)
+    W.close()
+
+
 def test_graph_capture_refuses_what_allocates_or_synchronises(lutgemm, oracle, device):
     """Under graph capture a stream's first launch on a handle (it would allocate the stream's set),
     the autotune calls and the workspace reset return LUTGEMM_ERR_UNSUPPORTED before any HIP call
