@@ -359,9 +359,11 @@ size_t workspace_bytes(const lutgemm_weight *w)
 // The set launches on `stream` use.  The first launch of a stream on this handle claims one.  The
 // caller holds the set (a lease) until release_set: launches are issued outside the lock, and a set
 // that another host thread is about to launch on must not be handed to a further stream meanwhile.
-int stream_set_once(lutgemm_weight *w, void *stream, int *slot, bool *leased_elsewhere)
+constexpr int kSetsLeased = -1;   // internal: nothing to take over only because other calls hold their sets right now
+
+int stream_set_once(lutgemm_weight *w, void *stream, int *slot, bool last_attempt)
 {
-    *leased_elsewhere = false;
+    bool leased_elsewhere = false;
     std::lock_guard<std::mutex> lock(w->slot_mutex);
     for (int i = 0; i < w->slots_used; i++)
         if (w->set[i].stream == stream) {
@@ -391,7 +393,7 @@ int stream_set_once(lutgemm_weight *w, void *stream, int *slot, bool *leased_els
         int idle = -1, busy = -1;
         for (int i = 0; i < kStreamSlots; i++) {
             const StreamSet &t = w->set[i];
-            if (t.leases > 0) *leased_elsewhere = true;
+            if (t.leases > 0) leased_elsewhere = true;
             if (!t.done_valid || t.leases > 0) continue;
             if (hipEventQuery(t.done) == hipSuccess) {
                 if (idle < 0 || t.last_use < w->set[idle].last_use) idle = i;
@@ -401,12 +403,18 @@ int stream_set_once(lutgemm_weight *w, void *stream, int *slot, bool *leased_els
         }
         (void)hipGetLastError();  // hipErrorNotReady from the queries is not a failure
         take = idle >= 0 ? idle : busy;
+        if (take < 0 && leased_elsewhere && !last_attempt) return kSetsLeased;
         if (take < 0)
             return fail(LUTGEMM_ERR_UNSUPPORTED,
                         "%d streams use this handle and none of their sets can be taken over (launches under "
                         "graph capture are not tracked); use lutgemm_weight_clone for further streams or "
                         "lutgemm_weight_reset_workspace to release the sets", kStreamSlots);
         if (idle < 0) {
+            if (stream_capturing(stream))   // a captured stream cannot wait for work outside its graph
+                return fail(LUTGEMM_ERR_UNSUPPORTED,
+                            "%d other streams are still using this handle's sets and a stream under graph capture "
+                            "cannot wait for them: launch once on the stream before capturing, or give it a handle "
+                            "of its own (lutgemm_weight_clone)", kStreamSlots);
             hipError_t e = hipStreamWaitEvent(static_cast<hipStream_t>(stream), w->set[take].done, 0);
             if (e != hipSuccess) return hip_fail(e, "hipStreamWaitEvent");
         }
@@ -423,10 +431,10 @@ int stream_set(lutgemm_weight *w, void *stream, int *slot)
 {
     // A lease lasts as long as another host thread needs to issue its launches: when that is all that
     // stands in the way of a take-over, try again shortly instead of failing.
+    constexpr int kAttempts = 200000;
     for (int attempt = 0;; attempt++) {
-        bool leased_elsewhere = false;
-        const int st = stream_set_once(w, stream, slot, &leased_elsewhere);
-        if (st != LUTGEMM_ERR_UNSUPPORTED || !leased_elsewhere || attempt >= 200000) return st;
+        const int st = stream_set_once(w, stream, slot, attempt + 1 >= kAttempts);
+        if (st != kSetsLeased) return st;
         std::this_thread::yield();
     }
 }
