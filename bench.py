@@ -328,6 +328,17 @@ def run_single(args, lutgemm, synth, torch, dev, stream, name):
     if args.copy_calibration:
         copy_calibration(torch, dev)
 
+    if name == "cfg1":
+        # what the box gives an ordinary device-to-device copy of 1 GiB, timed like everything else
+        src = torch.empty(512 * 1024 * 1024, dtype=torch.float16, device=dev).fill_(1.0)
+        dst = torch.empty_like(src)
+        prewarm(torch, lambda: dst.copy_(src))
+        cms = median(time_bursts(torch, stream, [lambda: dst.copy_(src)] * BURSTS))
+        line["measured_device_copy"] = {
+            "what": "torch device-to-device copy of 1 GiB on the same box (1 GiB read + 1 GiB written)",
+            "us": cms * 1e3, "GBps_read_plus_written": 2.0 * src.numel() * 2 / (cms * 1e-3) / 1e9}
+        del src, dst
+
     dense = None
     if name == "cfg1" and not args.no_dense:
         # dense fp16 GEMV of the same shape through the vendor library (rocBLAS/hipBLASLt via torch)
